@@ -1,0 +1,245 @@
+"""ctypes binding of libcutt.so: the four plan functions of include/cutt.h and
+the hooks of include/cutt_ext.h, with the same names and argument order.
+
+Device buffers are passed as integer addresses (e.g. ``tensor.data_ptr()``),
+streams as integer ``hipStream_t`` values (e.g.
+``torch.cuda.current_stream().cuda_stream``).  There is no CPU fallback: if
+the library is missing the import of :func:`lib` fails.
+"""
+import ctypes
+import os
+
+import numpy as np
+
+CUTT_SUCCESS = 0
+CUTT_INVALID_PLAN = 1
+CUTT_INVALID_PARAMETER = 2
+CUTT_INVALID_DEVICE = 3
+CUTT_INTERNAL_ERROR = 4
+CUTT_UNDEFINED_ERROR = 5
+_RESULT_NAMES = ["CUTT_SUCCESS", "CUTT_INVALID_PLAN", "CUTT_INVALID_PARAMETER", "CUTT_INVALID_DEVICE",
+                 "CUTT_INTERNAL_ERROR", "CUTT_UNDEFINED_ERROR"]
+
+METHOD_TRIVIAL, METHOD_PACKED, METHOD_PACKEDSPLIT, METHOD_TILED, METHOD_TILEDCOPY = 1, 2, 3, 4, 5
+METHOD_NAMES = {0: "Unknown", 1: "Trivial", 2: "Packed", 3: "PackedSplit", 4: "Tiled", 5: "TiledCopy"}
+
+
+class CuttError(RuntimeError):
+    def __init__(self, code, what):
+        name = _RESULT_NAMES[code] if 0 <= code < len(_RESULT_NAMES) else str(code)
+        super().__init__("%s returned %s" % (what, name))
+        self.code = code
+
+
+class PlanInfo(ctypes.Structure):
+    """Mirror of struct cuttPlanInfo (include/cutt_ext.h)."""
+    _fields_ = [
+        ("method", ctypes.c_int), ("fromReduced", ctypes.c_int), ("rank", ctypes.c_int),
+        ("numMm", ctypes.c_int), ("numMk", ctypes.c_int),
+        ("splitRank", ctypes.c_int), ("splitDim", ctypes.c_int), ("numSplit", ctypes.c_int),
+        ("volMm", ctypes.c_longlong), ("volMk", ctypes.c_longlong), ("volMmk", ctypes.c_longlong),
+        ("volMbar", ctypes.c_longlong), ("volMmkInCont", ctypes.c_longlong),
+        ("volMmkOutCont", ctypes.c_longlong), ("volMmkUnsplit", ctypes.c_longlong),
+        ("numBlocks", ctypes.c_longlong), ("numThreads", ctypes.c_int), ("itemsPerBlock", ctypes.c_int),
+        ("tiledOrder", ctypes.c_int), ("ldsBytes", ctypes.c_ulonglong),
+        ("usPredicted", ctypes.c_double),
+        ("rdLines", ctypes.c_double), ("wrLines", ctypes.c_double), ("rdInstr", ctypes.c_double),
+        ("wrInstr", ctypes.c_double), ("wrPartialLines", ctypes.c_double), ("rdSectors", ctypes.c_double),
+        ("wrSectors", ctypes.c_double), ("ldsCycles", ctypes.c_double), ("blocksPerCU", ctypes.c_double),
+        ("usMeasured", ctypes.c_double),
+        ("numCandidates", ctypes.c_int), ("planMs", ctypes.c_double),
+    ]
+
+    @property
+    def method_name(self):
+        return METHOD_NAMES.get(self.method, "?")
+
+    def as_dict(self):
+        d = {name: getattr(self, name) for name, _ in self._fields_}
+        d["method_name"] = self.method_name
+        return d
+
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_lib = None
+
+
+def lib_path():
+    return os.path.join(_HERE, "libcutt.so")
+
+
+def lib():
+    """Load libcutt.so (built in-tree by cutt_amd.build.build())."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = lib_path()
+    if not os.path.exists(path):
+        raise ImportError("%s not found: build it with `python -c 'import cutt_amd; cutt_amd.build()'`" % path)
+    l = ctypes.CDLL(path)
+    ip = ctypes.POINTER(ctypes.c_int)
+    hp = ctypes.POINTER(ctypes.c_uint)
+    vp = ctypes.c_void_p
+    l.cuttPlan.argtypes = [hp, ctypes.c_int, ip, ip, ctypes.c_size_t, vp]
+    l.cuttPlan.restype = ctypes.c_int
+    l.cuttPlanMeasure.argtypes = [hp, ctypes.c_int, ip, ip, ctypes.c_size_t, vp, vp, vp]
+    l.cuttPlanMeasure.restype = ctypes.c_int
+    l.cuttPlanFromCandidate.argtypes = [hp, ctypes.c_int, ip, ip, ctypes.c_size_t, vp, ctypes.c_int]
+    l.cuttPlanFromCandidate.restype = ctypes.c_int
+    l.cuttExecute.argtypes = [ctypes.c_uint, vp, vp]
+    l.cuttExecute.restype = ctypes.c_int
+    l.cuttDestroy.argtypes = [ctypes.c_uint]
+    l.cuttDestroy.restype = ctypes.c_int
+    l.cuttGetPlanInfo.argtypes = [ctypes.c_uint, ctypes.POINTER(PlanInfo)]
+    l.cuttGetPlanInfo.restype = ctypes.c_int
+    l.cuttSetMethodOverride.argtypes = [ctypes.c_int]
+    l.cuttSetMethodOverride.restype = None
+    l.cuttGetMethodOverride.argtypes = []
+    l.cuttGetMethodOverride.restype = ctypes.c_int
+    l.cuttGetLastMeasurement.argtypes = [ctypes.POINTER(PlanInfo), ctypes.c_int]
+    l.cuttGetLastMeasurement.restype = ctypes.c_int
+    l.cuttReduceRanks.argtypes = [ctypes.c_int, ip, ip, ip, ip]
+    l.cuttReduceRanks.restype = ctypes.c_int
+    l.cuttCandidatesCreate.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t]
+    l.cuttCandidatesCreate.restype = vp
+    l.cuttCandidatesCreateEx.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t, ctypes.c_size_t]
+    l.cuttCandidatesCreateEx.restype = vp
+    l.cuttCandidatesFree.argtypes = [vp]
+    l.cuttCandidatesFree.restype = None
+    l.cuttCandidatesCount.argtypes = [vp]
+    l.cuttCandidatesCount.restype = ctypes.c_int
+    l.cuttCandidatesBest.argtypes = [vp]
+    l.cuttCandidatesBest.restype = ctypes.c_int
+    l.cuttCandidatesInfo.argtypes = [vp, ctypes.c_int, ctypes.POINTER(PlanInfo)]
+    l.cuttCandidatesInfo.restype = ctypes.c_int
+    l.cuttCandidatesData.argtypes = [vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+                                     ctypes.POINTER(ctypes.c_longlong), ctypes.c_longlong]
+    l.cuttCandidatesData.restype = ctypes.c_longlong
+    l.cuttModelGlTransactionsSeg.argtypes = [ip, ctypes.c_int]
+    l.cuttModelGlTransactionsSeg.restype = ctypes.c_int
+    l.cuttModelGlTransactionsCont.argtypes = [ctypes.c_int] * 3
+    l.cuttModelGlTransactionsCont.restype = ctypes.c_int
+    l.cuttModelCacheLinesSeg.argtypes = [ip, ctypes.c_int, ctypes.c_int, ip, ip]
+    l.cuttModelCacheLinesSeg.restype = None
+    l.cuttModelCacheLinesCont.argtypes = [ctypes.c_int] * 3 + [ip, ip]
+    l.cuttModelCacheLinesCont.restype = None
+    l.cuttModelShTransactions.argtypes = [ctypes.c_int] * 4 + [ip, ctypes.c_int, ip]
+    l.cuttModelShTransactions.restype = None
+    _lib = l
+    return l
+
+
+def _ints(v):
+    return (ctypes.c_int * len(v))(*[int(x) for x in v])
+
+
+def _ptr(p):
+    return ctypes.c_void_p(int(p) if p else 0)
+
+
+def cuttPlan(rank, dim, permutation, sizeofType, stream=0):
+    """cuttPlan: returns (result code, handle)."""
+    h = ctypes.c_uint(0xFFFFFFFF)
+    rc = lib().cuttPlan(ctypes.byref(h), int(rank), _ints(dim), _ints(permutation), int(sizeofType), _ptr(stream))
+    return rc, h.value
+
+
+def cuttPlanMeasure(rank, dim, permutation, sizeofType, stream, idata, odata):
+    """cuttPlanMeasure: returns (result code, handle).  Destroys the contents of odata."""
+    h = ctypes.c_uint(0xFFFFFFFF)
+    rc = lib().cuttPlanMeasure(ctypes.byref(h), int(rank), _ints(dim), _ints(permutation), int(sizeofType),
+                               _ptr(stream), _ptr(idata), _ptr(odata))
+    return rc, h.value
+
+
+def cuttPlanFromCandidate(rank, dim, permutation, sizeofType, stream, index):
+    """Plan built from candidate `index` of the enumeration: returns (result code, handle)."""
+    h = ctypes.c_uint(0xFFFFFFFF)
+    rc = lib().cuttPlanFromCandidate(ctypes.byref(h), int(rank), _ints(dim), _ints(permutation),
+                                     int(sizeofType), _ptr(stream), int(index))
+    return rc, h.value
+
+
+def cuttExecute(handle, idata, odata):
+    return lib().cuttExecute(ctypes.c_uint(handle), _ptr(idata), _ptr(odata))
+
+
+def cuttDestroy(handle):
+    return lib().cuttDestroy(ctypes.c_uint(handle))
+
+
+def get_plan_info(handle):
+    info = PlanInfo()
+    rc = lib().cuttGetPlanInfo(ctypes.c_uint(handle), ctypes.byref(info))
+    if rc != CUTT_SUCCESS:
+        raise CuttError(rc, "cuttGetPlanInfo")
+    return info
+
+
+def set_method_override(method):
+    lib().cuttSetMethodOverride(int(method))
+
+
+def get_last_measurement():
+    n = lib().cuttGetLastMeasurement(None, 0)
+    arr = (PlanInfo * max(n, 1))()
+    lib().cuttGetLastMeasurement(arr, n)
+    return [arr[i] for i in range(n)]
+
+
+def reduce_ranks(dim, permutation):
+    n = len(dim)
+    rd = (ctypes.c_int * n)()
+    rp = (ctypes.c_int * n)()
+    k = lib().cuttReduceRanks(n, _ints(dim), _ints(permutation), rd, rp)
+    if k < 0:
+        raise ValueError("cuttReduceRanks failed")
+    return list(rd[:k]), list(rp[:k])
+
+
+class Candidates:
+    """The planner's candidate list for a problem, built for MI355X properties without a GPU."""
+
+    def __init__(self, dim, permutation, sizeofType, lds_per_block=0):
+        self._l = lib().cuttCandidatesCreateEx(len(dim), _ints(dim), _ints(permutation), int(sizeofType),
+                                               int(lds_per_block))
+        if not self._l:
+            raise ValueError("invalid transpose problem")
+
+    def close(self):
+        if self._l:
+            lib().cuttCandidatesFree(self._l)
+            self._l = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *a):
+        self.close()
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def __len__(self):
+        return lib().cuttCandidatesCount(self._l)
+
+    @property
+    def best(self):
+        return lib().cuttCandidatesBest(self._l)
+
+    def info(self, i):
+        info = PlanInfo()
+        if lib().cuttCandidatesInfo(self._l, i, ctypes.byref(info)) != 0:
+            raise IndexError(i)
+        return info
+
+    def data(self, i, what, cls=0):
+        n = lib().cuttCandidatesData(self._l, i, what, cls, None, 0)
+        if n < 0:
+            raise ValueError("no such data: candidate %d what %d" % (i, what))
+        buf = (ctypes.c_longlong * max(n, 1))()
+        lib().cuttCandidatesData(self._l, i, what, cls, buf, n)
+        return np.frombuffer(buf, dtype=np.int64, count=n).copy()

@@ -1,0 +1,499 @@
+/*
+ * cutt_api.cpp - the exported plan API (cutt.h) and its test hooks
+ * (cutt_ext.h): input validation, handle table, heuristic and measured plan
+ * selection.  Pure host C++; the GPU is reached through hip_layer.h.
+ *
+ * Mirrors the behaviour of reference src/cutt.cpp:36-310.  Deliberate
+ * differences: the handle table is guarded by a mutex (the reference's
+ * globals are unguarded, src/cutt.cpp:36-42); a HIP failure becomes
+ * CUTT_INTERNAL_ERROR instead of exit(1) (reference src/CudaUtils.h:35-42);
+ * cuttPlanMeasure times each candidate twice and keeps the faster run,
+ * because a first launch also pays for loading the kernel.
+ */
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include "../../include/cutt_ext.h"
+#include "hip_layer.h"
+#include "model.h"
+#include "plan.h"
+
+using namespace cutt;
+
+namespace {
+
+struct StoredPlan {
+  Plan plan;
+  int numCandidates = 0;
+  double planMs = 0;
+  double usMeasured = 0;
+};
+
+std::mutex gMutex;
+std::unordered_map<cuttHandle, StoredPlan*> gPlans;
+cuttHandle gNextHandle = 0;
+std::unordered_map<int, cuttHipDeviceProps> gDeviceProps;
+int gMethodOverride = -1;  // -1 = not initialised from the environment yet
+std::vector<cuttPlanInfo> gLastMeasurement;
+
+int methodOverrideLocked() {
+  if (gMethodOverride < 0) {
+    gMethodOverride = 0;
+    const char* e = std::getenv("CUTT_FORCE_METHOD");
+    if (e) {
+      std::string s(e);
+      for (char& c : s) c = (char)std::tolower((unsigned char)c);
+      if (s == "tiled") gMethodOverride = kTiled;
+      else if (s == "tiledcopy") gMethodOverride = kTiledCopy;
+      else if (s == "packed") gMethodOverride = kPacked;
+      else if (s == "packedsplit") gMethodOverride = kPackedSplit;
+    }
+  }
+  return gMethodOverride;
+}
+
+// Same checks as reference src/cutt.cpp:59-82, plus the 2^31 element limit that the
+// reference's int arithmetic implies.
+cuttResult checkInput(int rank, const int* dim, const int* perm, size_t sizeofType) {
+  if (sizeofType != 4 && sizeofType != 8) return CUTT_INVALID_PARAMETER;
+  if (rank <= 1 || rank > CUTT_MAX_RANK) return CUTT_INVALID_PARAMETER;
+  if (!dim || !perm) return CUTT_INVALID_PARAMETER;
+  long long vol = 1;
+  for (int i = 0; i < rank; i++) {
+    if (dim[i] <= 1) return CUTT_INVALID_PARAMETER;
+    vol *= dim[i];
+    if (vol >= (1ll << 31)) return CUTT_INVALID_PARAMETER;
+  }
+  std::vector<char> seen(rank, 0);
+  for (int i = 0; i < rank; i++) {
+    if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) return CUTT_INVALID_PARAMETER;
+    seen[perm[i]] = 1;
+  }
+  return CUTT_SUCCESS;
+}
+
+bool currentDevice(int& deviceID, cuttHipDeviceProps& props) {
+  if (cuttHipGetDevice(&deviceID) != 0) return false;
+  std::lock_guard<std::mutex> lock(gMutex);
+  auto it = gDeviceProps.find(deviceID);
+  if (it == gDeviceProps.end()) {
+    cuttHipDeviceProps p;
+    if (cuttHipGetDeviceProps(deviceID, &p) != 0) return false;
+    it = gDeviceProps.emplace(deviceID, p).first;
+  }
+  props = it->second;
+  return true;
+}
+
+void fillInfo(const Plan& p, cuttPlanInfo& o) {
+  std::memset(&o, 0, sizeof(o));
+  o.method = p.method;
+  o.fromReduced = p.fromReduced;
+  o.rank = p.pb.rank;
+  o.numMm = p.split.numMm;
+  o.numMk = p.split.numMk;
+  o.splitRank = p.split.splitRank;
+  o.splitDim = p.split.splitDim;
+  o.numSplit = p.split.numSplit;
+  o.volMm = p.split.volMm;
+  o.volMk = p.split.volMk;
+  o.volMmk = p.split.volMmk;
+  o.volMbar = p.split.volMbar;
+  o.volMmkInCont = p.split.volMmkInCont;
+  o.volMmkOutCont = p.split.volMmkOutCont;
+  o.volMmkUnsplit = p.split.volMmkUnsplit;
+  o.numBlocks = p.numBlocks;
+  o.numThreads = p.numThreads;
+  o.itemsPerBlock = p.packed.itemsPerBlock;
+  o.tiledOrder = p.method == kTiled ? p.tiled.order : p.tcopy.order;
+  o.ldsBytes = p.ldsBytes;
+  o.usPredicted = p.model.usPredicted;
+  o.rdLines = p.model.rdLines;
+  o.wrLines = p.model.wrLines;
+  o.rdInstr = p.model.rdInstr;
+  o.wrInstr = p.model.wrInstr;
+  o.wrPartialLines = p.model.wrPartialLines;
+  o.rdSectors = p.model.rdSectors;
+  o.wrSectors = p.model.wrSectors;
+  o.ldsCycles = p.model.ldsCycles;
+  o.blocksPerCU = p.model.blocksPerCU;
+}
+
+// Index of the candidate with the smallest predicted time; Trivial always wins and ties go to
+// the later candidate (reference src/cuttplan.cpp:700-768).
+int chooseHeuristic(const std::vector<Plan>& plans) {
+  int best = -1;
+  for (int i = 0; i < (int)plans.size(); i++) {
+    if (plans[i].method == kTrivial) return i;
+    if (best < 0 || plans[i].model.usPredicted <= plans[best].model.usPredicted) best = i;
+  }
+  return best;
+}
+
+bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
+               const cuttHipDeviceProps& props, int forceMethod, std::vector<Plan>& plans) {
+  Problem orig, red;
+  orig.set(rank, dim, perm, (int)sizeofType);
+  std::vector<int> redDim, redPerm;
+  reduceRanks(rank, dim, perm, redDim, redPerm);
+  red.set((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType);
+  PlannerOptions opt;
+  opt.forceMethod = forceMethod;
+  return createPlans(orig, red, props, opt, plans);
+}
+
+cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int deviceID, int numCandidates,
+                     double usMeasured, std::chrono::steady_clock::time_point t0) {
+  StoredPlan* sp = new StoredPlan();
+  sp->plan = std::move(chosen);
+  sp->plan.stream = stream;
+  sp->plan.deviceID = deviceID;
+  sp->numCandidates = numCandidates;
+  sp->usMeasured = usMeasured;
+  if (sp->plan.activate() != 0) {
+    delete sp;
+    return CUTT_INTERNAL_ERROR;
+  }
+  sp->planMs = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  std::lock_guard<std::mutex> lock(gMutex);
+  *handle = gNextHandle++;
+  if (gPlans.count(*handle)) {
+    delete sp;
+    return CUTT_INTERNAL_ERROR;
+  }
+  gPlans.emplace(*handle, sp);
+  return CUTT_SUCCESS;
+}
+
+}  // namespace
+
+extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
+                               size_t sizeofType, hipStream_t stream) {
+  const auto t0 = std::chrono::steady_clock::now();
+  if (!handle) return CUTT_INVALID_PARAMETER;
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  if (chk != CUTT_SUCCESS) return chk;
+
+  int deviceID;
+  cuttHipDeviceProps props;
+  if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  std::vector<Plan> plans;
+  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
+  for (Plan& p : plans)
+    if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
+  const int best = chooseHeuristic(plans);
+  if (best < 0) return CUTT_INTERNAL_ERROR;
+  return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
+}
+
+extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                      size_t sizeofType, hipStream_t stream, void* idata, void* odata) {
+  const auto t0 = std::chrono::steady_clock::now();
+  if (!handle) return CUTT_INVALID_PARAMETER;
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  if (chk != CUTT_SUCCESS) return chk;
+  if (idata == odata || !idata || !odata) return CUTT_INVALID_PARAMETER;
+
+  int deviceID;
+  cuttHipDeviceProps props;
+  if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  std::vector<Plan> plans;
+  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
+  if (plans.empty()) return CUTT_INTERNAL_ERROR;
+  // The model's numbers are kept for reporting; they do not influence the choice.
+  for (Plan& p : plans)
+    if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
+
+  size_t numBytes = sizeofType;
+  for (int i = 0; i < rank; i++) numBytes *= (size_t)dim[i];
+
+  void *evStart = nullptr, *evStop = nullptr;
+  if (cuttHipEventCreate(&evStart) != 0) return CUTT_INTERNAL_ERROR;
+  if (cuttHipEventCreate(&evStop) != 0) {
+    cuttHipEventDestroy(evStart);
+    return CUTT_INTERNAL_ERROR;
+  }
+  std::vector<double> us(plans.size(), 0.0);
+  int best = -1;
+  double bestUs = 1e300;
+  bool failed = false;
+  for (int i = 0; i < (int)plans.size() && !failed; i++) {
+    Plan& p = plans[i];
+    p.stream = (void*)stream;
+    p.deviceID = deviceID;
+    if (p.activate() != 0) { failed = true; break; }
+    double t = 1e300;
+    for (int rep = 0; rep < 2; rep++) {
+      // Overwrite the output so that every run starts from the same cache state.
+      if (cuttHipMemsetAsync(odata, 0xFF, numBytes, (void*)stream) != 0 ||
+          cuttHipDeviceSynchronize() != 0 || cuttHipEventRecord(evStart, (void*)stream) != 0 ||
+          p.launch(idata, odata) != 0 || cuttHipEventRecord(evStop, (void*)stream) != 0 ||
+          cuttHipEventSynchronize(evStop) != 0) {
+        failed = true;
+        break;
+      }
+      float ms = 0;
+      if (cuttHipEventElapsedMs(evStart, evStop, &ms) != 0) { failed = true; break; }
+      t = std::min(t, (double)ms * 1e3);
+      if (t > 3.0 * bestUs) break;  // hopeless: do not spend a second run on it
+    }
+    us[i] = t;
+    if (!failed && t < bestUs) {
+      bestUs = t;
+      best = i;
+    }
+    if (i != best) p.release();
+    // a previous best that has been beaten no longer needs its tables
+    for (int j = 0; j < i; j++)
+      if (j != best) plans[j].release();
+  }
+  cuttHipEventDestroy(evStart);
+  cuttHipEventDestroy(evStop);
+  if (failed || best < 0) return CUTT_INTERNAL_ERROR;
+
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    gLastMeasurement.resize(plans.size());
+    for (size_t i = 0; i < plans.size(); i++) {
+      fillInfo(plans[i], gLastMeasurement[i]);
+      gLastMeasurement[i].usMeasured = us[i];
+      gLastMeasurement[i].numCandidates = (int)plans.size();
+    }
+  }
+  return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), bestUs, t0);
+}
+
+extern "C" cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                            size_t sizeofType, hipStream_t stream, int index) {
+  const auto t0 = std::chrono::steady_clock::now();
+  if (!handle) return CUTT_INVALID_PARAMETER;
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  if (chk != CUTT_SUCCESS) return chk;
+  int deviceID;
+  cuttHipDeviceProps props;
+  if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  std::vector<Plan> plans;
+  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
+  if (index < 0 || index >= (int)plans.size()) return CUTT_INVALID_PARAMETER;
+  if (!estimatePlan(plans[index], props, 10)) return CUTT_INTERNAL_ERROR;
+  return storePlan(handle, std::move(plans[index]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
+}
+
+extern "C" cuttResult cuttDestroy(cuttHandle handle) {
+  StoredPlan* sp = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    auto it = gPlans.find(handle);
+    if (it == gPlans.end()) return CUTT_INVALID_PLAN;
+    sp = it->second;
+    gPlans.erase(it);
+  }
+  delete sp;
+  return CUTT_SUCCESS;
+}
+
+extern "C" cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata) {
+  StoredPlan* sp = nullptr;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    auto it = gPlans.find(handle);
+    if (it == gPlans.end()) return CUTT_INVALID_PLAN;
+    sp = it->second;
+  }
+  if (idata == odata || !idata || !odata) return CUTT_INVALID_PARAMETER;
+  int deviceID;
+  if (cuttHipGetDevice(&deviceID) != 0) return CUTT_INTERNAL_ERROR;
+  if (deviceID != sp->plan.deviceID) return CUTT_INVALID_DEVICE;
+  if (sp->plan.launch(idata, odata) != 0) return CUTT_INTERNAL_ERROR;
+  return CUTT_SUCCESS;
+}
+
+// ---------------------------------------------------------------------------
+// cutt_ext.h
+// ---------------------------------------------------------------------------
+extern "C" cuttResult cuttGetPlanInfo(cuttHandle handle, cuttPlanInfo* info) {
+  if (!info) return CUTT_INVALID_PARAMETER;
+  std::lock_guard<std::mutex> lock(gMutex);
+  auto it = gPlans.find(handle);
+  if (it == gPlans.end()) return CUTT_INVALID_PLAN;
+  fillInfo(it->second->plan, *info);
+  info->numCandidates = it->second->numCandidates;
+  info->planMs = it->second->planMs;
+  info->usMeasured = it->second->usMeasured;
+  return CUTT_SUCCESS;
+}
+
+extern "C" void cuttSetMethodOverride(int method) {
+  std::lock_guard<std::mutex> lock(gMutex);
+  gMethodOverride = (method > 0 && method < kNumMethods) ? method : 0;
+}
+
+extern "C" int cuttGetMethodOverride(void) {
+  std::lock_guard<std::mutex> lock(gMutex);
+  return methodOverrideLocked();
+}
+
+extern "C" int cuttGetLastMeasurement(cuttPlanInfo* infos, int maxInfos) {
+  std::lock_guard<std::mutex> lock(gMutex);
+  const int n = (int)gLastMeasurement.size();
+  for (int i = 0; i < n && i < maxInfos && infos; i++) infos[i] = gLastMeasurement[i];
+  return n;
+}
+
+extern "C" int cuttReduceRanks(int rank, const int* dim, const int* permutation, int* redDim,
+                               int* redPermutation) {
+  if (rank < 1 || !dim || !permutation || !redDim || !redPermutation) return -1;
+  std::vector<int> d, p;
+  reduceRanks(rank, dim, permutation, d, p);
+  for (size_t i = 0; i < d.size(); i++) {
+    redDim[i] = d[i];
+    redPermutation[i] = p[i];
+  }
+  return (int)d.size();
+}
+
+namespace {
+struct CandidateList {
+  std::vector<Plan> plans;
+  int best = -1;
+};
+}  // namespace
+
+extern "C" void* cuttCandidatesCreateEx(int rank, const int* dim, const int* permutation,
+                                        size_t sizeofType, size_t ldsPerBlock) {
+  if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS) return nullptr;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  CandidateList* l = new CandidateList();
+  cuttHipDeviceProps props = defaultMI355XProps();
+  if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
+  if (!enumerate(rank, dim, permutation, sizeofType, props, force, l->plans)) {
+    delete l;
+    return nullptr;
+  }
+  for (Plan& p : l->plans) {
+    if (!p.buildTables() || !estimatePlan(p, props, 10)) {
+      delete l;
+      return nullptr;
+    }
+  }
+  l->best = chooseHeuristic(l->plans);
+  return l;
+}
+
+extern "C" void* cuttCandidatesCreate(int rank, const int* dim, const int* permutation,
+                                      size_t sizeofType) {
+  return cuttCandidatesCreateEx(rank, dim, permutation, sizeofType, 0);
+}
+
+extern "C" void cuttCandidatesFree(void* list) { delete (CandidateList*)list; }
+extern "C" int cuttCandidatesCount(void* list) { return list ? (int)((CandidateList*)list)->plans.size() : -1; }
+extern "C" int cuttCandidatesBest(void* list) { return list ? ((CandidateList*)list)->best : -1; }
+
+extern "C" int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info) {
+  CandidateList* l = (CandidateList*)list;
+  if (!l || !info || index < 0 || index >= (int)l->plans.size()) return -1;
+  fillInfo(l->plans[index], *info);
+  info->numCandidates = (int)l->plans.size();
+  return 0;
+}
+
+extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
+                                        long long maxCount) {
+  CandidateList* l = (CandidateList*)list;
+  if (!l || index < 0 || index >= (int)l->plans.size() || cls < 0 || cls > 1) return -1;
+  const Plan& p = l->plans[index];
+  std::vector<long long> v;
+  const bool packed = p.method == kPacked || p.method == kPackedSplit;
+  switch (what) {
+    case 0: {
+      const cuttHipMbar& mb = packed ? p.packed.mbar : (p.method == kTiled ? p.tiled.mbar : p.tcopy.mbar);
+      if (p.method == kTrivial) break;
+      for (int k = 0; k < mb.n; k++) {
+        v.push_back(mb.d[k].extent);
+        v.push_back(mb.d[k].strideIn);
+        v.push_back(mb.d[k].strideOut);
+      }
+    } break;
+    case 1:
+      if (p.method == kTiled)
+        v = {p.tiled.volMm, p.tiled.volMk, p.tiled.strideInK, p.tiled.strideOutM, p.tiled.tilesM,
+             p.tiled.tilesK, p.tiled.volMbar, p.tiled.order};
+      else if (p.method == kTiledCopy)
+        v = {p.tcopy.volMm, p.tcopy.volMk, p.tcopy.strideInK, p.tcopy.strideOutK, p.tcopy.tilesM,
+             p.tcopy.tilesK, p.tcopy.volMbar, p.tcopy.order};
+      else
+        return -1;
+      break;
+    case 2:
+      if (!packed) return -1;
+      v = {p.packed.numThreads, p.packed.volMbar, p.packed.numSplit, p.packed.slabFloor,
+           p.packed.slabRem, p.packed.splitStrideIn, p.packed.splitStrideOut, p.packed.itemsPerBlock,
+           p.packed.padShift, p.packed.ldsElems};
+      break;
+    case 3: {
+      if (!packed) return -1;
+      const cuttHipPackedClass& k = p.packed.cls[cls];
+      v = {k.vol, k.inCont, k.outCont, k.inMagic, k.outMagic, k.nRowsIn, k.nRowsOut};
+    } break;
+    case 4:
+      if (!packed) return -1;
+      v.assign(p.tab[cls].rowIn.begin(), p.tab[cls].rowIn.end());
+      break;
+    case 5:
+      if (!packed) return -1;
+      v.assign(p.tab[cls].rowOut.begin(), p.tab[cls].rowOut.end());
+      break;
+    case 6:
+      if (!packed) return -1;
+      v.assign(p.tab[cls].shIdx.begin(), p.tab[cls].shIdx.end());
+      break;
+    default:
+      return -1;
+  }
+  for (long long i = 0; i < (long long)v.size() && i < maxCount && values; i++) values[i] = v[(size_t)i];
+  return (long long)v.size();
+}
+
+extern "C" int cuttModelGlTransactionsSeg(const int* seg, int n) { return glTransactions(seg, n); }
+extern "C" int cuttModelGlTransactionsCont(int pos, int n, int accWidth) {
+  return glTransactions(pos, n, accWidth);
+}
+extern "C" void cuttModelCacheLinesSeg(const int* seg, int n, int cacheWidth, int* clFull, int* clPart) {
+  countCacheLines(seg, n, cacheWidth, *clFull, *clPart);
+}
+extern "C" void cuttModelCacheLinesCont(int pos, int n, int cacheWidth, int* clFull, int* clPart) {
+  countCacheLines(pos, n, cacheWidth, *clFull, *clPart);
+}
+extern "C" void cuttModelShTransactions(int waveSize, int numBanks, int numThreads, int volMmk,
+                                        const int* msh, int numMsh, int* out4) {
+  std::vector<ShConv> m(numMsh);
+  for (int i = 0; i < numMsh; i++) m[i] = {msh[3 * i], msh[3 * i + 1], msh[3 * i + 2]};
+  out4[0] = out4[1] = out4[2] = out4[3] = 0;
+  countShTransactions(waveSize, numBanks, numThreads, volMmk, m.data(), numMsh, out4[0], out4[1],
+                      out4[2], out4[3]);
+}

@@ -1,0 +1,169 @@
+/*
+ * hip_layer.h - the thin C-ABI layer between the host planner and HIP.
+ *
+ * Everything above this header (cutt_api.cpp, plan.cpp, model.cpp) is plain
+ * host C++ that never includes a HIP header; everything that touches the HIP
+ * runtime or contains device code lives behind these functions
+ * (hip_layer.hip, kernels.hip).  All arguments are plain C types; a stream or
+ * event travels as void*.  Every function returns 0 on success or the
+ * hipError_t value on failure (cuttHipErrorString turns it into text).
+ *
+ * It takes the place of three pieces of the reference: the kernel interface
+ * src/cuttkernel.h:29-34 (launch configuration + cuttKernel), the device
+ * helpers src/CudaUtils.h:44-122 (allocate/copy/memset wrappers) and the
+ * event timer src/cuttTimer.h:46-61.
+ */
+#ifndef CUTT_HIP_LAYER_H
+#define CUTT_HIP_LAYER_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Largest tensor rank the kernels accept (the per-rank tables travel as kernel arguments). */
+#define CUTT_MAX_RANK 32
+
+/* Device facts the planner and the cost model need. */
+typedef struct cuttHipDeviceProps {
+  int cuCount;              /* compute units */
+  int waveSize;             /* lanes per wavefront (64 on gfx950) */
+  int maxThreadsPerBlock;
+  int maxThreadsPerCU;
+  size_t ldsPerBlock;       /* bytes of LDS one workgroup may allocate */
+  size_t ldsPerCU;          /* bytes of LDS per compute unit */
+  int clockKHz;             /* shader clock */
+  int memClockKHz;
+  int memBusWidthBits;
+  int l2Bytes;
+  int maxGridX;
+  char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
+} cuttHipDeviceProps;
+
+/*
+ * One rank of the "remaining" index set (Mbar): the ranks that neither the
+ * input-contiguous set nor the output-contiguous set of a plan covers.  A
+ * workgroup's position m in that set is decomposed as
+ *   i_k = m % extent_k, m /= extent_k   (ranks in input order)
+ * and contributes i_k*strideIn to the input offset and i_k*strideOut to the
+ * output offset (offsets in elements).
+ */
+typedef struct cuttHipMbarDim {
+  uint32_t extent;
+  uint32_t strideIn;
+  uint32_t strideOut;
+} cuttHipMbarDim;
+
+typedef struct cuttHipMbar {
+  int n;
+  cuttHipMbarDim d[CUTT_MAX_RANK];
+} cuttHipMbar;
+
+/*
+ * Tiled method: a batch of 2-D transposes between input rank 0 (extent volMm,
+ * input stride 1, output stride strideOutM) and the rank that leads the
+ * output (extent volMk, input stride strideInK, output stride 1), staged
+ * through a padded 64x64 LDS tile.  One workgroup per (tile, Mbar position).
+ */
+typedef struct cuttHipTiledArgs {
+  int elemSize;       /* 4 or 8 */
+  int volMm, volMk;
+  uint32_t strideInK;
+  uint32_t strideOutM;
+  int tilesM, tilesK; /* ceil(volMm/64), ceil(volMk/64) */
+  int volMbar;
+  int order;          /* workgroup-index decoding: 0 = Mbar fastest, 1 = tiles along Mm fastest, 2 = tiles along Mk fastest */
+  cuttHipMbar mbar;
+} cuttHipTiledArgs;
+
+/*
+ * TiledCopy method: rank 0 keeps its place, so rows along rank 0 (extent
+ * volMm) are copied; the second output rank (extent volMk, input stride
+ * strideInK, output stride strideOutK) is the other tile axis.  No LDS.
+ */
+typedef struct cuttHipTiledCopyArgs {
+  int elemSize;
+  int volMm, volMk;
+  uint32_t strideInK;
+  uint32_t strideOutK;
+  int tilesM, tilesK;
+  int volMbar;
+  int order;
+  cuttHipMbar mbar;
+} cuttHipTiledCopyArgs;
+
+/*
+ * Index tables of a Packed / PackedSplit plan for one slab size (device
+ * pointers).  The staged block holds `vol` elements.  In input-compact order
+ * element p lies in row p / inCont at column p % inCont, and is read from
+ * input offset rowIn[row] + column; it is stored in LDS slot
+ * p + (p >> padShift).  In output-compact order element q is written to
+ * output offset rowOut[q / outCont] + q % outCont and taken from LDS slot
+ * shIdx[q] (padding included).  inMagic/outMagic = ceil(2^32 / inCont|outCont)
+ * for the multiply-high division.
+ */
+typedef struct cuttHipPackedClass {
+  int vol;
+  int inCont, outCont;
+  uint32_t inMagic, outMagic;
+  int nRowsIn, nRowsOut;
+  const uint32_t* rowIn;
+  const uint32_t* rowOut;
+  const uint16_t* shIdx;
+} cuttHipPackedClass;
+
+/*
+ * Packed and PackedSplit methods.  Work items are (Mbar position m, slab s),
+ * numbered w = m*numSplit + s; workgroup b handles items
+ * [b*itemsPerBlock, (b+1)*itemsPerBlock).  Slab s covers
+ * [s*slabFloor + min(s, slabRem), ...) of the split rank and has
+ * slabFloor + (s < slabRem) entries: class 1 if s < slabRem, else class 0.
+ * Packed is the case numSplit == 1 (one slab of class 0, no split rank).
+ */
+typedef struct cuttHipPackedArgs {
+  int elemSize;
+  int numThreads;
+  int volMbar;
+  int numSplit;
+  int slabFloor, slabRem;
+  uint32_t splitStrideIn, splitStrideOut; /* global strides of the split rank */
+  int itemsPerBlock;
+  int padShift;        /* LDS slot(p) = p + (p >> padShift); 31 = no padding */
+  int ldsElems;        /* element slots in the LDS data buffer (padding included) */
+  int maxRowsIn, maxRowsOut, maxVol; /* maxima over the classes: LDS table sizes */
+  cuttHipPackedClass cls[2];
+  cuttHipMbar mbar;
+} cuttHipPackedArgs;
+
+/* Bytes of LDS the packed kernel needs for these arguments. */
+size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a);
+
+/* ---- device, memory, stream and event helpers ---------------------------- */
+int cuttHipGetDevice(int* device);
+int cuttHipGetDeviceProps(int device, cuttHipDeviceProps* props);
+int cuttHipMalloc(void** ptr, size_t bytes);
+int cuttHipFree(void* ptr);
+/* Host to device copy that has completed when the call returns. */
+int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes);
+int cuttHipMemcpyDtoDAsync(void* dst, const void* src, size_t bytes, void* stream);
+int cuttHipMemsetAsync(void* dst, int value, size_t bytes, void* stream);
+int cuttHipDeviceSynchronize(void);
+int cuttHipEventCreate(void** event);
+int cuttHipEventDestroy(void* event);
+int cuttHipEventRecord(void* event, void* stream);
+int cuttHipEventSynchronize(void* event);
+int cuttHipEventElapsedMs(void* start, void* stop, float* ms);
+const char* cuttHipErrorString(int err);
+
+/* ---- kernel launches (asynchronous on `stream`) -------------------------- */
+int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
+int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
+int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CUTT_HIP_LAYER_H */

@@ -1,0 +1,316 @@
+/*
+ * model.cpp - memory-transaction cost model.  See model.h.
+ *
+ * The counting functions keep the reference's definitions (reference
+ * src/cuttGpuModel.cpp:52-204, 477-559) so that its known-answer tables still
+ * apply; the widths are parameters.  The plan estimate is new: it walks the
+ * address stream of the gfx950 kernels in kernels.hip (64 lanes per request,
+ * 128-byte lines, 32-byte sectors, 64x64 tiles, row/column packed tables).
+ */
+#include "model.h"
+
+#include <algorithm>
+#include <cmath>
+#include <random>
+#include <vector>
+
+namespace cutt {
+
+int glTransactions(const int* seg, int n) {
+  if (n <= 0) return 0;
+  int count = 1;
+  for (int i = 1; i < n; i++) count += (seg[i] != seg[i - 1]);
+  return count;
+}
+
+int glTransactions(int pos, int n, int accWidth) {
+  if (n <= 0) return 0;
+  return (pos + n - 1) / accWidth - pos / accWidth + 1;
+}
+
+void countCacheLines(const int* seg, int n, int cacheWidth, int& clFull, int& clPart) {
+  // Positions increase monotonically, so the lanes that touch one line are a run of equal
+  // segment numbers; the line is fully covered when the run has cacheWidth members.
+  clFull = clPart = 0;
+  int i = 0;
+  while (i < n) {
+    int j = i + 1;
+    while (j < n && seg[j] == seg[i]) j++;
+    if (j - i >= cacheWidth)
+      clFull++;
+    else
+      clPart++;
+    i = j;
+  }
+}
+
+void countCacheLines(int pos, int n, int cacheWidth, int& clFull, int& clPart) {
+  clFull = clPart = 0;
+  if (n <= 0) return;
+  const int first = pos / cacheWidth, last = (pos + n - 1) / cacheWidth;
+  const bool headPartial = (pos % cacheWidth) != 0;
+  const bool tailPartial = ((pos + n) % cacheWidth) != 0;
+  if (first == last) {
+    if (headPartial || tailPartial) clPart = 1; else clFull = 1;
+    return;
+  }
+  clPart = (int)headPartial + (int)tailPartial;
+  clFull = (last - first + 1) - clPart;
+}
+
+void countShTransactions(int waveSize, int numBanks, int numThreads, int volMmk, const ShConv* msh,
+                         int numMsh, int& sldTran, int& sstTran, int& sldReq, int& sstReq) {
+  std::vector<int> perBank(numBanks);
+  for (int blockStart = 0; blockStart < volMmk; blockStart += numThreads) {
+    const int blockEnd = std::min(volMmk, blockStart + numThreads);
+    for (int w0 = blockStart; w0 < blockEnd; w0 += waveSize) {
+      const int n = std::min(waveSize, volMmk - w0);
+      std::fill(perBank.begin(), perBank.end(), 0);
+      int degree = 0;
+      for (int l = 0; l < n; l++) {
+        const int j = w0 + l;
+        int pos = 0;
+        for (int k = 0; k < numMsh; k++) pos += ((j / msh[k].c) % msh[k].d) * msh[k].ct;
+        degree = std::max(degree, ++perBank[pos % numBanks]);
+      }
+      sldTran += degree;
+      sstTran += 1;
+      sldReq += 1;
+      sstReq += 1;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+namespace {
+
+constexpr int kTile = 64;
+constexpr int kLineBytes = 128;
+constexpr int kSectorBytes = 32;
+constexpr int kLdsBanks = 64;
+
+struct Counts {
+  double rdLines = 0, wrLines = 0, rdInstr = 0, wrInstr = 0, wrPartial = 0, rdSectors = 0,
+         wrSectors = 0, ldsCycles = 0;
+  void add(const Counts& o, double w) {
+    rdLines += w * o.rdLines; wrLines += w * o.wrLines; rdInstr += w * o.rdInstr;
+    wrInstr += w * o.wrInstr; wrPartial += w * o.wrPartial; rdSectors += w * o.rdSectors;
+    wrSectors += w * o.wrSectors; ldsCycles += w * o.ldsCycles;
+  }
+};
+
+// A contiguous run of n elements at element offset pos: lines, sectors, partial lines.
+inline void runCost(int64_t pos, int64_t n, int es, double& lines, double& sectors, double& partial) {
+  if (n <= 0) return;
+  const int64_t b0 = pos * es, b1 = (pos + n) * es;  // [b0, b1)
+  const int64_t l0 = b0 / kLineBytes, l1 = (b1 - 1) / kLineBytes;
+  lines += (double)(l1 - l0 + 1);
+  sectors += (double)((b1 - 1) / kSectorBytes - b0 / kSectorBytes + 1);
+  const bool head = (b0 % kLineBytes) != 0, tail = (b1 % kLineBytes) != 0;
+  if (l0 == l1) partial += (head || tail) ? 1 : 0;
+  else partial += (int)head + (int)tail;
+}
+
+void mbarOffsets(const cuttHipMbar& mb, uint32_t m, int64_t& offIn, int64_t& offOut) {
+  offIn = offOut = 0;
+  for (int k = 0; k < mb.n; k++) {
+    const uint32_t i = m % mb.d[k].extent;
+    m /= mb.d[k].extent;
+    offIn += (int64_t)i * mb.d[k].strideIn;
+    offOut += (int64_t)i * mb.d[k].strideOut;
+  }
+}
+
+// One tile of w x h elements (w along rank 0, h along the Mk rank).
+Counts tileCost(bool copy, int es, int64_t offIn, int64_t offOut, int64_t m0, int64_t k0, int w, int h,
+                int64_t strideInK, int64_t strideOut) {
+  Counts c;
+  double dummy = 0;
+  for (int k = 0; k < h; k++) {
+    runCost(offIn + m0 + (k0 + k) * strideInK, w, es, c.rdLines, c.rdSectors, dummy);
+    c.rdInstr += 1;
+  }
+  if (copy) {
+    for (int k = 0; k < h; k++) {
+      runCost(offOut + m0 + (k0 + k) * strideOut, w, es, c.wrLines, c.wrSectors, c.wrPartial);
+      c.wrInstr += 1;
+    }
+  } else {
+    for (int m = 0; m < w; m++) {
+      runCost(offOut + k0 + (m0 + m) * strideOut, h, es, c.wrLines, c.wrSectors, c.wrPartial);
+      c.wrInstr += 1;
+    }
+    // LDS: one padded-tile write and one read per element row, conflict free.
+    c.ldsCycles += (double)(h + w) * (es == 8 ? 4 : 2);
+  }
+  return c;
+}
+
+Counts tiledSample(const Plan& p, bool copy, uint32_t m) {
+  const int es = p.pb.elemSize;
+  const int volMm = copy ? p.tcopy.volMm : p.tiled.volMm;
+  const int volMk = copy ? p.tcopy.volMk : p.tiled.volMk;
+  const int64_t sIn = copy ? p.tcopy.strideInK : p.tiled.strideInK;
+  const int64_t sOut = copy ? p.tcopy.strideOutK : p.tiled.strideOutM;
+  int64_t offIn, offOut;
+  mbarOffsets(copy ? p.tcopy.mbar : p.tiled.mbar, m, offIn, offOut);
+  const int fullM = volMm / kTile, fullK = volMk / kTile;
+  const int remM = volMm % kTile, remK = volMk % kTile;
+  Counts total;
+  if (fullM && fullK)
+    total.add(tileCost(copy, es, offIn, offOut, 0, 0, kTile, kTile, sIn, sOut), (double)fullM * fullK);
+  if (remM && fullK)
+    total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, 0, remM, kTile, sIn, sOut), fullK);
+  if (remK && fullM)
+    total.add(tileCost(copy, es, offIn, offOut, 0, (int64_t)fullK * kTile, kTile, remK, sIn, sOut), fullM);
+  if (remM && remK)
+    total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, (int64_t)fullK * kTile, remM, remK,
+                       sIn, sOut), 1);
+  return total;
+}
+
+// One staged block of a Packed / PackedSplit plan.
+Counts packedSample(const Plan& p, int cls, int64_t offIn, int64_t offOut) {
+  const int es = p.pb.elemSize;
+  const PackedTables& t = p.tab[cls];
+  Counts c;
+  std::vector<int64_t> lines;
+  lines.reserve(128);
+  // Reads: wavefront requests cover 64 consecutive input-compact positions.
+  for (int p0 = 0; p0 < t.vol; p0 += 64) {
+    const int p1 = std::min(t.vol, p0 + 64);
+    lines.clear();
+    double sectors = 0;
+    int q = p0;
+    while (q < p1) {
+      const int row = q / t.inCont, col = q % t.inCont;
+      const int n = std::min(p1 - q, t.inCont - col);
+      const int64_t pos = offIn + t.rowIn[row] + col;
+      const int64_t b0 = pos * es, b1 = (pos + n) * es;
+      for (int64_t l = b0 / kLineBytes; l <= (b1 - 1) / kLineBytes; l++) lines.push_back(l);
+      sectors += (double)((b1 - 1) / kSectorBytes - b0 / kSectorBytes + 1);
+      q += n;
+    }
+    std::sort(lines.begin(), lines.end());
+    c.rdLines += (double)(std::unique(lines.begin(), lines.end()) - lines.begin());
+    c.rdSectors += sectors;
+    c.rdInstr += 1;
+  }
+  // Writes: 64 consecutive output-compact positions per request.
+  std::vector<int> bank(kLdsBanks);
+  for (int q0 = 0; q0 < t.vol; q0 += 64) {
+    const int q1 = std::min(t.vol, q0 + 64);
+    lines.clear();
+    double sectors = 0;
+    int q = q0;
+    while (q < q1) {
+      const int row = q / t.outCont, col = q % t.outCont;
+      const int n = std::min(q1 - q, t.outCont - col);
+      const int64_t pos = offOut + t.rowOut[row] + col;
+      const int64_t b0 = pos * es, b1 = (pos + n) * es;
+      for (int64_t l = b0 / kLineBytes; l <= (b1 - 1) / kLineBytes; l++) lines.push_back(l);
+      sectors += (double)((b1 - 1) / kSectorBytes - b0 / kSectorBytes + 1);
+      q += n;
+    }
+    std::sort(lines.begin(), lines.end());
+    c.wrLines += (double)(std::unique(lines.begin(), lines.end()) - lines.begin());
+    c.wrSectors += sectors;
+    c.wrInstr += 1;
+    // LDS gather: conflict degree over 4-byte banks; 8-byte words occupy two banks.
+    std::fill(bank.begin(), bank.end(), 0);
+    int degree = 0;
+    const int words = es / 4;
+    for (int k = q0; k < q1; k++) degree = std::max(degree, ++bank[(t.shIdx[k] * words) % kLdsBanks]);
+    c.ldsCycles += (double)degree * words + words;  // gather read + linear write
+  }
+  // Partial lines of the output rows (each row is one contiguous run).
+  for (size_t r = 0; r < t.rowOut.size(); r++) {
+    double l = 0, s = 0;
+    runCost(offOut + t.rowOut[r], t.outCont, es, l, s, c.wrPartial);
+  }
+  return c;
+}
+
+}  // namespace
+
+bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
+  ModelResult& r = plan.model;
+  r = ModelResult();
+  const int es = plan.pb.elemSize;
+  const double bytes = (double)plan.pb.volume * es;
+  if (plan.method == kTrivial) {
+    r.rdLines = r.wrLines = bytes / kLineBytes;
+    r.rdSectors = r.wrSectors = bytes / kSectorBytes;
+    r.usPredicted = 0.0;  // a plain copy always wins (reference src/cuttplan.cpp:705-707)
+    return true;
+  }
+  std::minstd_rand0 rng;  // fixed seed: deterministic plans
+  Counts total;
+  double tableBytes = 0;
+  if (plan.method == kTiled || plan.method == kTiledCopy) {
+    const bool copy = plan.method == kTiledCopy;
+    const uint32_t volMbar = (uint32_t)plan.split.volMbar;
+    const int ns = (numSamples == 0 || (uint32_t)numSamples > volMbar) ? (int)volMbar : numSamples;
+    std::uniform_int_distribution<uint32_t> pick(0, volMbar - 1);
+    for (int i = 0; i < ns; i++) {
+      const uint32_t m = ((uint32_t)ns == volMbar) ? (uint32_t)i : pick(rng);
+      total.add(tiledSample(plan, copy, m), (double)volMbar / ns);
+    }
+  } else {
+    if (!plan.buildTables()) return false;
+    const cuttHipPackedArgs& a = plan.packed;
+    const uint32_t items = (uint32_t)a.volMbar * (uint32_t)a.numSplit;
+    const int ns = (numSamples == 0 || (uint32_t)numSamples > items) ? (int)items : numSamples;
+    std::uniform_int_distribution<uint32_t> pick(0, items - 1);
+    for (int i = 0; i < ns; i++) {
+      const uint32_t w = ((uint32_t)ns == items) ? (uint32_t)i : pick(rng);
+      const uint32_t m = w / a.numSplit, s = w % a.numSplit;
+      const int cls = s < (uint32_t)a.slabRem ? 1 : 0;
+      const int64_t p0 = (int64_t)s * a.slabFloor + std::min<int64_t>(s, a.slabRem);
+      int64_t offIn, offOut;
+      mbarOffsets(a.mbar, m, offIn, offOut);
+      offIn += p0 * a.splitStrideIn;
+      offOut += p0 * a.splitStrideOut;
+      total.add(packedSample(plan, cls, offIn, offOut), (double)items / ns);
+    }
+    // Every workgroup loads its tables once from L2.
+    tableBytes = (double)plan.numBlocks * (2.0 * a.maxVol + 4.0 * (a.maxRowsIn + a.maxRowsOut));
+  }
+  r.rdLines = total.rdLines; r.wrLines = total.wrLines;
+  r.rdInstr = total.rdInstr; r.wrInstr = total.wrInstr;
+  r.wrPartialLines = total.wrPartial;
+  r.rdSectors = total.rdSectors; r.wrSectors = total.wrSectors;
+  r.ldsCycles = total.ldsCycles;
+
+  // Resident workgroups per CU.
+  const double byLds = plan.ldsBytes ? std::floor((double)props.ldsPerCU / (double)plan.ldsBytes) : 32.0;
+  const double byThreads = std::floor((double)props.maxThreadsPerCU / plan.numThreads);
+  const double blocksPerCU = std::max(1.0, std::min({byLds, byThreads, 32.0}));
+  r.blocksPerCU = blocksPerCU;
+
+  // --- time estimate ---
+  const double clockHz = props.clockKHz * 1e3;
+  const double cus = props.cuCount;
+  // Sustained HBM traffic: what a large device-to-device copy reaches on this part.
+  const double peakBW = (double)props.memClockKHz * 1e3 * 4.0 * (props.memBusWidthBits / 8.0);
+  const double sustainedBW = 0.64 * peakBW;
+  // Reads move whole lines; writes move the touched sectors, partial lines pay a merge penalty.
+  const double traffic = r.rdLines * kLineBytes + r.wrSectors * kSectorBytes +
+                         r.wrPartialLines * 64.0 + 0.25 * tableBytes;
+  const double tMem = traffic / sustainedBW;
+  // Address processing: a request costs at least 4 cycles, or one cycle per line it touches.
+  const double reqCycles = std::max(4.0 * (r.rdInstr + r.wrInstr), r.rdLines + r.wrLines);
+  const double tReq = reqCycles / (cus * clockHz);
+  const double tLds = r.ldsCycles / (cus * clockHz);
+  // Latency bound: bytes in flight per CU (4 loads per lane) against ~2 us loaded latency.
+  const double lanes = std::min((double)props.maxThreadsPerCU, blocksPerCU * plan.numThreads);
+  const double inflight = 0.5 * lanes * 4.0 * es * cus;  // half the waves are in their store phase
+  const double tLat = bytes / (inflight / 2.0e-6);
+  // Workgroup launch + barrier overhead.
+  const double tBlocks = (double)plan.numBlocks * 1.5e-6 / (cus * blocksPerCU);
+  const double t = std::max({tMem, tReq, tLat}) + 0.5 * tLds + tBlocks;
+  r.usPredicted = t * 1e6;
+  return true;
+}
+
+}  // namespace cutt

@@ -1,0 +1,140 @@
+/*
+ * plan.h - host-side planner: rank fusing, index-set splits, candidate
+ * enumeration, index tables and launch geometry.  Pure host C++; the device is
+ * reached only through hip_layer.h.
+ *
+ * Counterpart of reference src/cuttplan.h:36-212 (method enum, TensorSplit,
+ * LaunchConfig, cuttPlan_t) with a different organisation: a candidate owns
+ * the ready-to-launch kernel arguments, and Packed tables are compact
+ * (one offset per contiguous row + a 16-bit LDS gather index per element).
+ */
+#ifndef CUTT_PLAN_H
+#define CUTT_PLAN_H
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "hip_layer.h"
+
+namespace cutt {
+
+// Same numbering as the reference's method enum (src/cuttplan.h:37-39).
+enum Method { kUnknown = 0, kTrivial = 1, kPacked = 2, kPackedSplit = 3, kTiled = 4, kTiledCopy = 5, kNumMethods };
+
+const char* methodName(int method);
+
+// A transpose problem: dims (dim[0] fastest), permutation, element size, strides.
+struct Problem {
+  int rank = 0;
+  int elemSize = 0;
+  std::vector<int> dim;
+  std::vector<int> perm;       // output rank j is input rank perm[j]
+  std::vector<int> inv;        // inv[perm[j]] = j
+  std::vector<int64_t> strideIn;   // input stride of input rank r
+  std::vector<int64_t> strideOut;  // output stride of input rank r
+  int64_t volume = 0;
+
+  void set(int rank, const int* dim, const int* perm, int elemSize);
+};
+
+// Fuse runs of ranks that stay adjacent and in order (reference src/cuttplan.cpp:63-126).
+void reduceRanks(int rank, const int* dim, const int* perm, std::vector<int>& redDim,
+                 std::vector<int>& redPerm);
+
+/*
+ * How a candidate divides the ranks (vocabulary of reference src/cuttplan.h:41-82):
+ *   Mm   = the first numMm input ranks,  Mk = the first numMk output ranks,
+ *   Mmk  = Mm u Mk (staged by one workgroup), Mbar = everything else.
+ */
+struct Split {
+  int method = kUnknown;
+  int numMm = 0, numMk = 0;
+  int sizeMmk = 0, sizeMbar = 0, sizeMkBar = 0;
+  int64_t volMm = 0, volMk = 0, volMmk = 0, volMkBar = 0, volMbar = 0;
+  int64_t volMmkInCont = 0, volMmkOutCont = 0;  // for the largest slab when split
+  // PackedSplit
+  int splitRank = -1;
+  int splitDim = 0;
+  int numSplit = 1;
+  int64_t volMmkUnsplit = 0;
+  std::vector<char> inMmk;  // per input rank
+
+  void update(int numMm, int numMk, const Problem& pb);
+  int slabMax() const { return splitRank < 0 ? 0 : (splitDim + numSplit - 1) / numSplit; }
+  int64_t volStaged() const;  // elements one workgroup stages at most
+};
+
+// Host copy of the index tables of one slab size (see cuttHipPackedClass).
+struct PackedTables {
+  int vol = 0, inCont = 0, outCont = 0;
+  std::vector<uint32_t> rowIn, rowOut;
+  std::vector<uint16_t> shIdx;
+};
+
+// Counters and estimate produced by the cost model (model.h).
+struct ModelResult {
+  double rdLines = 0, wrLines = 0;     // 128-byte lines touched, whole tensor
+  double rdInstr = 0, wrInstr = 0;     // wavefront-level memory instructions, whole tensor
+  double wrPartialLines = 0;           // written lines not fully covered by one workgroup
+  double rdSectors = 0, wrSectors = 0; // 32-byte sectors touched
+  double ldsCycles = 0;                // LDS cycles incl. bank conflicts, whole tensor
+  double blocksPerCU = 0;
+  double usPredicted = 0;              // predicted time in microseconds (ranking key)
+};
+
+struct Plan {
+  int method = kUnknown;
+  Split split;
+  Problem pb;             // the problem this candidate was built from (original or fused)
+  bool fromReduced = false;
+  int deviceID = -1;
+  void* stream = nullptr;
+
+  cuttHipTiledArgs tiled;
+  cuttHipTiledCopyArgs tcopy;
+  cuttHipPackedArgs packed;
+  size_t ldsBytes = 0;
+  int64_t numBlocks = 0;
+  int numThreads = 0;
+
+  // Packed host tables, built on demand (buildTables) and device copies (activate).
+  PackedTables tab[2];
+  bool tablesBuilt = false;
+  void* dTables = nullptr;
+
+  ModelResult model;
+
+  Plan();
+  ~Plan();
+  Plan(const Plan&) = delete;
+  Plan& operator=(const Plan&) = delete;
+  Plan(Plan&& o) noexcept;
+  Plan& operator=(Plan&& o) noexcept;
+
+  bool buildTables();             // Packed/PackedSplit: fill tab[]; others: no-op
+  int activate();                 // upload tables; returns 0 or a HIP error code
+  int launch(const void* in, void* out);  // asynchronous on stream
+  void release();                 // free device tables
+  std::string describe() const;
+};
+
+struct PlannerOptions {
+  int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
+  int tiledOrder = -1;      // -1 = planner's choice
+};
+
+// Build every candidate for the original and the fused problem
+// (reference src/cuttplan.cpp:681-698).  Returns false on an internal error.
+bool createPlans(const Problem& orig, const Problem& red, const cuttHipDeviceProps& props,
+                 const PlannerOptions& opt, std::vector<Plan>& plans);
+
+// Default device description of one MI355X, used when no GPU is present (tests, offline planning).
+cuttHipDeviceProps defaultMI355XProps();
+
+// magic = ceil(2^32 / d) for the multiply-high division used by the packed kernel (d >= 2).
+uint32_t divMagic(uint32_t d);
+
+}  // namespace cutt
+
+#endif  // CUTT_PLAN_H

@@ -1,0 +1,93 @@
+/*
+ * cutt.h - tensor transpose plan API for AMD Instinct MI355X (gfx950).
+ *
+ * Drop-in for the plan API of cuTT: the four entry points, the handle type and
+ * the result enum keep the names, argument order, argument meaning and enum
+ * values of the reference header (reference src/cutt.h:31-41, 57-58, 76-77,
+ * 88, 101); the only change in the signatures is hipStream_t where the
+ * reference has cudaStream_t.  The symbols have C linkage, so the library can
+ * be bound from C, C++ (source compatible with callers of the reference
+ * header) and any FFI.
+ *
+ * Conventions (reference README.md:78-125):
+ *   - dim[0] is the fastest running (contiguous) dimension of the input;
+ *   - output dimension j is input dimension permutation[j], i.e. the output
+ *     tensor has dimensions dim[permutation[0]], dim[permutation[1]], ...;
+ *   - elements are opaque 4- or 8-byte values, moved bit-exactly;
+ *   - transposes are out-of-place; idata and odata must not overlap;
+ *   - dim and permutation are host arrays, read during the call only.
+ */
+#ifndef CUTT_H
+#define CUTT_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Same definition as in <hip/hip_runtime_api.h>; repeating a typedef is legal. */
+typedef struct ihipStream_t* hipStream_t;
+
+/* Handle that names a plan (reference src/cutt.h:31). */
+typedef unsigned int cuttHandle;
+
+/* Return values, same order and values as reference src/cutt.h:34-41. */
+typedef enum cuttResult_t {
+  CUTT_SUCCESS,            /* Success */
+  CUTT_INVALID_PLAN,       /* Invalid plan handle */
+  CUTT_INVALID_PARAMETER,  /* Invalid input parameter */
+  CUTT_INVALID_DEVICE,     /* Execution tried on device different than where plan was created */
+  CUTT_INTERNAL_ERROR,     /* Internal error */
+  CUTT_UNDEFINED_ERROR     /* Undefined error */
+} cuttResult;
+
+/*
+ * Create a plan; the method is chosen by the cost model.
+ * Replaces reference cuttPlan (src/cutt.h:57-58, src/cutt.cpp:84-184).
+ *
+ *   handle            returned plan handle
+ *   rank              rank of the tensor (>= 2)
+ *   dim[rank]         dimensions, every one >= 2
+ *   permutation[rank] a permutation of 0..rank-1
+ *   sizeofType        element size in bytes, 4 or 8
+ *   stream            HIP stream the plan executes on (0 = default stream)
+ *
+ * The plan is bound to the device that is current at the call.
+ */
+cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
+                    size_t sizeofType, hipStream_t stream);
+
+/*
+ * Create a plan; every candidate is run on idata/odata, timed with HIP events,
+ * and the fastest is kept.  Replaces reference cuttPlanMeasure
+ * (src/cutt.h:76-77, src/cutt.cpp:186-284).
+ *
+ *   idata, odata      device buffers of product(dim)*sizeofType bytes.
+ *                     The contents of odata are destroyed.
+ *
+ * Synchronises the device.
+ */
+cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, int* permutation,
+                           size_t sizeofType, hipStream_t stream, void* idata, void* odata);
+
+/*
+ * Destroy a plan and free its device tables.  Replaces reference cuttDestroy
+ * (src/cutt.h:88, src/cutt.cpp:286-294).  The caller makes sure that no
+ * execution of the plan is still in flight.
+ */
+cuttResult cuttDestroy(cuttHandle handle);
+
+/*
+ * Execute a plan out-of-place, asynchronously on the plan's stream.  Replaces
+ * reference cuttExecute (src/cutt.h:101, src/cutt.cpp:296-310).
+ *
+ *   idata, odata      device buffers of product(dim)*sizeofType bytes
+ */
+cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CUTT_H */

@@ -1,0 +1,137 @@
+/*
+ * cutt_ext.h - introspection and test hooks beside the four plan functions of
+ * cutt.h.  None of these has a counterpart in the reference's public header;
+ * they expose what the reference only prints (cuttPlan_t::print,
+ * src/cuttplan.cpp:792-809), what its test driver reaches through internal
+ * headers (testCounters, src/cuttGpuModel.h:85; reduceRanks,
+ * src/cuttplan.h:215-216), and an override that pins the method so that each
+ * kernel can be measured alone.
+ */
+#ifndef CUTT_EXT_H
+#define CUTT_EXT_H
+
+#include "cutt.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Method numbers, as in the reference's enum (src/cuttplan.h:37-39). */
+enum {
+  CUTT_METHOD_UNKNOWN = 0,
+  CUTT_METHOD_TRIVIAL = 1,
+  CUTT_METHOD_PACKED = 2,
+  CUTT_METHOD_PACKEDSPLIT = 3,
+  CUTT_METHOD_TILED = 4,
+  CUTT_METHOD_TILEDCOPY = 5
+};
+
+/* What a plan (or a candidate) looks like. */
+typedef struct cuttPlanInfo {
+  int method;
+  int fromReduced;      /* 1 if built from the rank-fused problem */
+  int rank;             /* rank of the problem the plan was built from */
+  int numMm, numMk;
+  int splitRank, splitDim, numSplit;
+  long long volMm, volMk, volMmk, volMbar, volMmkInCont, volMmkOutCont, volMmkUnsplit;
+  long long numBlocks;
+  int numThreads;
+  int itemsPerBlock;    /* Packed/PackedSplit */
+  int tiledOrder;       /* Tiled/TiledCopy */
+  unsigned long long ldsBytes;
+  /* cost model */
+  double usPredicted;
+  double rdLines, wrLines, rdInstr, wrInstr, wrPartialLines, rdSectors, wrSectors, ldsCycles,
+      blocksPerCU;
+  /* filled by cuttPlanMeasure: time of this candidate's timed run, else 0 */
+  double usMeasured;
+  /* planning statistics of the call that made the plan */
+  int numCandidates;
+  double planMs;
+} cuttPlanInfo;
+
+/* Describe an existing plan. */
+cuttResult cuttGetPlanInfo(cuttHandle handle, cuttPlanInfo* info);
+
+/*
+ * Restrict the planner to one method (CUTT_METHOD_*; 0 = no restriction) for
+ * plans created afterwards by this process.  A transpose that fuses to a plain
+ * copy still yields a Trivial plan.  If the method has no feasible candidate,
+ * cuttPlan returns CUTT_INTERNAL_ERROR.  The environment variable
+ * CUTT_FORCE_METHOD (tiled, tiledcopy, packed, packedsplit) sets the initial
+ * value.
+ */
+void cuttSetMethodOverride(int method);
+int cuttGetMethodOverride(void);
+
+/*
+ * After cuttPlanMeasure: the candidates it timed, best first is NOT implied;
+ * they are in enumeration order.  Returns the number of candidates of the most
+ * recent cuttPlanMeasure call of this process and copies up to maxInfos
+ * descriptions.
+ */
+int cuttGetLastMeasurement(cuttPlanInfo* infos, int maxInfos);
+
+/*
+ * Create a plan from candidate number `index` of the planner's enumeration for
+ * this problem on the current device (0 <= index < numCandidates, see
+ * cuttPlanInfo.numCandidates; out of range -> CUTT_INVALID_PARAMETER).  Lets a
+ * test or a tuning run execute every candidate, not only the chosen one.
+ */
+cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                 size_t sizeofType, hipStream_t stream, int index);
+
+/* Fuse ranks that stay adjacent and ordered; returns the fused rank.
+ * redDim and redPermutation must hold `rank` entries. */
+int cuttReduceRanks(int rank, const int* dim, const int* permutation, int* redDim,
+                    int* redPermutation);
+
+/* ---- candidate lists without a GPU (tests, offline inspection) ----------- */
+
+/*
+ * Enumerate the candidates the planner would build for this problem on a
+ * device with MI355X properties (no GPU needed, nothing is launched).
+ * Returns an opaque list or NULL on invalid input; free it with
+ * cuttCandidatesFree.
+ */
+void* cuttCandidatesCreate(int rank, const int* dim, const int* permutation, size_t sizeofType);
+/* Same with a different LDS size per workgroup (0 = the device's), so that small test tensors
+ * also produce PackedSplit candidates. */
+void* cuttCandidatesCreateEx(int rank, const int* dim, const int* permutation, size_t sizeofType,
+                             size_t ldsPerBlock);
+void cuttCandidatesFree(void* list);
+int cuttCandidatesCount(void* list);
+/* Index of the candidate the cost model ranks best. */
+int cuttCandidatesBest(void* list);
+int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
+
+/*
+ * Raw index data of candidate `index`, for checking a plan's address stream
+ * on the host.  `what` selects the array, `cls` the slab class (0/1) where it
+ * applies; the function copies up to maxCount 64-bit values into `values` and
+ * returns the array's length (or -1).
+ *
+ *   what 0: Mbar table, 3 values per rank: extent, strideIn, strideOut
+ *   what 1: tile geometry: volMm, volMk, strideInK, strideOut(M or K), tilesM, tilesK, volMbar, order
+ *   what 2: packed scalars: numThreads, volMbar, numSplit, slabFloor, slabRem, splitStrideIn,
+ *           splitStrideOut, itemsPerBlock, padShift, ldsElems
+ *   what 3: class scalars: vol, inCont, outCont, inMagic, outMagic, nRowsIn, nRowsOut
+ *   what 4: rowIn[]   what 5: rowOut[]   what 6: shIdx[]
+ */
+long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
+                             long long maxCount);
+
+/* ---- counters of the cost model (known-answer tests) --------------------- */
+int cuttModelGlTransactionsSeg(const int* seg, int n);
+int cuttModelGlTransactionsCont(int pos, int n, int accWidth);
+void cuttModelCacheLinesSeg(const int* seg, int n, int cacheWidth, int* clFull, int* clPart);
+void cuttModelCacheLinesCont(int pos, int n, int cacheWidth, int* clFull, int* clPart);
+/* msh: numMsh triples (c, d, ct).  out: sldTran, sstTran, sldReq, sstReq. */
+void cuttModelShTransactions(int waveSize, int numBanks, int numThreads, int volMmk, const int* msh,
+                             int numMsh, int* out4);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* CUTT_EXT_H */

@@ -1,0 +1,137 @@
+"""Host planner: rank fusing, candidate enumeration and index tables (no GPU).
+
+Every candidate's address stream is replayed with numpy (plan_emulator.py) and
+compared with the CPU oracle, so table or geometry mistakes show up here
+before any kernel runs.
+"""
+import itertools
+
+import numpy as np
+import pytest
+
+from plan_emulator import emulate
+from test_oracle import REDUCE_CASES
+
+
+@pytest.mark.parametrize("dim,perm,rdim,rperm", REDUCE_CASES)
+def test_reduce_ranks_hand_cases(cutt, dim, perm, rdim, rperm):
+    assert cutt.reduce_ranks(dim, perm) == (rdim, rperm)
+
+
+def test_reduce_ranks_matches_oracle(cutt, oracle_mod):
+    rng = np.random.default_rng(1)
+    for _ in range(300):
+        rank = int(rng.integers(2, 16))
+        dim = [int(d) for d in rng.integers(2, 10, size=rank)]
+        perm = [int(p) for p in rng.permutation(rank)]
+        if rng.random() < 0.5:  # make fusable runs likely
+            perm = sorted(perm[: rank // 2]) + perm[rank // 2:]
+        assert cutt.reduce_ranks(dim, perm) == oracle_mod.reduce_ranks(dim, perm)
+
+
+def check_all_candidates(cutt, oracle_mod, dim, perm, es, lds=0, need=None):
+    dtype = np.uint32 if es == 4 else np.uint64
+    vol = int(np.prod(dim))
+    data = (np.arange(vol, dtype=np.uint64) * 2654435761 % (2 ** 31)).astype(dtype)
+    expect = oracle_mod.transpose(dim, perm, data)
+    seen = set()
+    with cutt.Candidates(dim, perm, es, lds) as c:
+        assert len(c) >= 1
+        assert 0 <= c.best < len(c)
+        for i in range(len(c)):
+            info = c.info(i)
+            seen.add(info.method_name)
+            out, count = emulate(c, i, data)
+            assert count.min() == 1 and count.max() == 1, (dim, perm, info.method_name, "write coverage")
+            assert np.array_equal(out, expect), (dim, perm, es, info.as_dict())
+    if need:
+        assert need in seen, (need, seen)
+    return seen
+
+
+@pytest.mark.parametrize("rank", [2, 3, 4, 5])
+def test_all_permutations_small(cutt, oracle_mod, rank):
+    # shapes of the reference's test1 (src/cutt_test.cpp:138-158): dim[r] = 2 + r*14/rank
+    dim = [2 + r * 14 // rank for r in range(rank)]
+    for perm in itertools.permutations(range(rank)):
+        for es in (4, 8):
+            check_all_candidates(cutt, oracle_mod, dim, perm, es)
+
+
+@pytest.mark.parametrize("rank", [6, 7])
+def test_sampled_permutations_rank67(cutt, oracle_mod, rank):
+    dim = [2 + r * 14 // rank for r in range(rank)]
+    rng = np.random.default_rng(rank)
+    for _ in range(6):
+        perm = [int(p) for p in rng.permutation(rank)]
+        check_all_candidates(cutt, oracle_mod, dim, perm, 8 if rng.random() < 0.5 else 4)
+
+
+def test_small_lds_forces_split(cutt, oracle_mod):
+    # With 2-4 KB of LDS even small tensors need PackedSplit, including uneven slabs.
+    rng = np.random.default_rng(2)
+    seen = set()
+    for _ in range(40):
+        rank = int(rng.integers(2, 6))
+        dim = [int(d) for d in rng.integers(2, 24, size=rank)]
+        perm = [int(p) for p in rng.permutation(rank)]
+        es = 4 if rng.random() < 0.5 else 8
+        seen |= check_all_candidates(cutt, oracle_mod, dim, perm, es, lds=int(rng.choice([1024, 2048, 4096])))
+    assert "PackedSplit" in seen and "Packed" in seen and "Tiled" in seen and "TiledCopy" in seen
+
+
+HAND_PICKED = [  # reference src/cutt_test.cpp:245-366 (test3), shrunk where the volume is large
+    ((43, 67), (1, 0), "Tiled"),
+    ((4099, 2), (1, 0), "Tiled"),
+    ((131, 59, 8), (0, 2, 1), "TiledCopy"),
+    ((24, 33, 8, 7), (1, 0, 2, 3), "Tiled"),
+    ((5, 12, 15, 16, 7), (1, 3, 4, 2, 0), "Packed"),
+    ((5, 3, 2, 9, 14), (0, 1, 3, 2, 4), "TiledCopy"),
+    ((24, 8, 4, 6, 7, 3), (5, 1, 4, 2, 3, 0), "Packed"),
+]
+
+
+@pytest.mark.parametrize("dim,perm,need", HAND_PICKED)
+def test_hand_picked(cutt, oracle_mod, dim, perm, need):
+    for es in (4, 8):
+        check_all_candidates(cutt, oracle_mod, dim, perm, es, need=need)
+
+
+def test_identity_gives_trivial(cutt):
+    for dim in [(2, 5, 9, 12), (2, 4, 6, 9, 11, 13)]:
+        with cutt.Candidates(dim, range(len(dim)), 8) as c:
+            assert len(c) == 1 and c.info(0).method_name == "Trivial"
+
+
+def test_invalid_problems_rejected(cutt):
+    for dim, perm, es in [((4, 4), (0, 0), 4), ((4, 1), (1, 0), 4), ((4, 4), (1, 0), 2), ((4,), (0,), 4),
+                          ((4, 4), (1, 2), 8), ((65536, 65536), (1, 0), 4)]:
+        with pytest.raises(ValueError):
+            cutt.Candidates(dim, perm, es)
+
+
+def method_set(cutt, dim, perm, es):
+    with cutt.Candidates(dim, perm, es) as c:
+        infos = [c.info(i) for i in range(len(c))]
+        return infos, infos[c.best]
+
+
+def test_baseline_configs_have_their_method(cutt):
+    # C1/C2: LDS-tiled kernel; C3: Packed; C4: PackedSplit must at least be available.
+    infos, best = method_set(cutt, (8192, 8192), (1, 0), 4)
+    assert any(i.method_name == "Tiled" for i in infos)
+    infos, best = method_set(cutt, (1024, 64, 1024, 3), (2, 1, 0, 3), 8)
+    t = [i for i in infos if i.method_name == "Tiled"]
+    assert len(t) == 1 and t[0].volMm == 1024 and t[0].volMk == 1024 and t[0].volMbar == 192
+    infos, best = method_set(cutt, (5, 7, 11, 13, 17, 1093), (4, 2, 0, 5, 1, 3), 4)
+    p = [i for i in infos if i.method_name == "Packed" and i.volMmk == 6545]
+    assert p and p[0].volMmkInCont == 385 and p[0].volMmkOutCont == 935 and p[0].volMbar == 14209
+    infos, best = method_set(cutt, (200000, 2, 500), (2, 1, 0), 8)
+    assert any(i.method_name == "PackedSplit" for i in infos)
+    assert any(i.method_name == "Tiled" and i.volMm == 200000 and i.volMk == 500 for i in infos)
+
+
+def test_plans_are_deterministic(cutt):
+    a = method_set(cutt, (31, 549, 2, 3), (3, 0, 2, 1), 8)
+    b = method_set(cutt, (31, 549, 2, 3), (3, 0, 2, 1), 8)
+    assert [i.as_dict() for i in a[0]] == [i.as_dict() for i in b[0]]
