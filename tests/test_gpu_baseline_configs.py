@@ -1,0 +1,109 @@
+"""The benchmark configurations at full size: bit-exact against the CPU oracle, plus
+size-independent properties (transpose followed by the inverse transpose is the identity;
+the plan's method does not change the bytes)."""
+import sys
+
+import numpy as np
+import pytest
+
+import baseline_configs as bc
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import gpu_util
+    import cutt_amd
+    cutt_amd.lib()
+    cutt_amd.set_method_override(0)
+    return gpu_util
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("cfg", bc.FIXED, ids=[c["name"] for c in bc.FIXED])
+def test_fixed_config_bit_exact(gpu, cfg):
+    import oracle
+    import torch
+    import cutt_amd as cutt
+    dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
+    data = bc.make_input(cfg)
+    say("%s: oracle on the host" % cfg["name"])
+    if cfg["name"] == "C1":
+        expect = oracle.transpose(dim, perm, data)   # single-thread index loop, as the config says
+    else:
+        expect = oracle.transpose_mt(dim, perm, data, 16)
+    for how in ("plan", "measure"):
+        say("%s: %s" % (cfg["name"], how))
+        info = gpu.check_case(dim, perm, es, data=data, how=how, expect=expect)
+        say("  -> %s blocks=%d threads=%d" % (info.method_name, info.numBlocks, info.numThreads))
+    # inverse round trip on the device
+    d_in = gpu.to_device(data)
+    d_mid = torch.empty_like(d_in)
+    d_back = torch.empty_like(d_in)
+    st = gpu.stream_handle()
+    odim = [dim[p] for p in perm]
+    inv = [perm.index(r) for r in range(len(perm))]
+    rc1, h1 = cutt.cuttPlan(len(dim), dim, perm, es, st)
+    rc2, h2 = cutt.cuttPlan(len(dim), odim, inv, es, st)
+    assert rc1 == 0 and rc2 == 0
+    gpu.run_plan(h1, d_in, d_mid)
+    gpu.run_plan(h2, d_mid, d_back)
+    assert torch.equal(d_back, d_in)
+    cutt.cuttDestroy(h1)
+    cutt.cuttDestroy(h2)
+
+
+def test_c4_forced_packed_split(gpu):
+    # C4 is the "packed-split case": the method is pinned so that this kernel runs at full size
+    import oracle
+    import cutt_amd as cutt
+    cfg = bc.C4
+    dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
+    data = bc.make_input(cfg)
+    expect = oracle.transpose_mt(dim, perm, data, 16)
+    try:
+        cutt.set_method_override(cutt.METHOD_PACKEDSPLIT)
+        for how in ("plan", "measure"):
+            info = gpu.check_case(dim, perm, es, data=data, how=how, expect=expect)
+            assert info.method == cutt.METHOD_PACKEDSPLIT
+            say("C4 forced PackedSplit (%s): numSplit=%d blocks=%d lds=%d" %
+                (how, info.numSplit, info.numBlocks, info.ldsBytes))
+    finally:
+        cutt.set_method_override(0)
+
+
+def test_sweep_sample_all_methods_agree(gpu):
+    # three tensors of the C5 sweep: every method the planner offers gives the same bytes
+    import torch
+    import cutt_amd as cutt
+    for cfg in bc.sweep()[:6:2]:
+        dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
+        data = bc.make_input(cfg, seed=99)
+        d_in = gpu.to_device(data)
+        st = gpu.stream_handle()
+        results = []
+        for method in (0, cutt.METHOD_TILED, cutt.METHOD_TILEDCOPY, cutt.METHOD_PACKED, cutt.METHOD_PACKEDSPLIT):
+            cutt.set_method_override(method)
+            try:
+                rc, h = cutt.cuttPlan(len(dim), dim, perm, es, st)
+            finally:
+                cutt.set_method_override(0)
+            if rc != cutt.CUTT_SUCCESS:
+                continue  # this method has no candidate for the shape
+            say("%s dim=%s perm=%s method %s" % (cfg["name"], dim, perm, cutt.get_plan_info(h).method_name))
+            d_out = torch.full_like(d_in, -1)
+            gpu.run_plan(h, d_in, d_out)
+            cutt.cuttDestroy(h)
+            results.append(d_out)
+        assert len(results) >= 2
+        for r in results[1:]:
+            assert torch.equal(r, results[0])
+        import oracle
+        assert np.array_equal(gpu.to_host(results[0], es), oracle.transpose_mt(dim, perm, data, 16))

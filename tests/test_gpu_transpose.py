@@ -1,0 +1,183 @@
+"""GPU parity tests: every transpose goes through the C-ABI (cuttPlan /
+cuttPlanMeasure / cuttExecute / cuttDestroy) and is compared bit-exact with
+the CPU oracle.  The shapes follow the reference's own test driver
+(reference src/cutt_test.cpp:138-431)."""
+import itertools
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    import gpu_util
+    import cutt_amd
+    cutt_amd.lib()  # fails loudly if libcutt.so is missing
+    cutt_amd.set_method_override(0)
+    return gpu_util
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.mark.parametrize("rank", [2, 3, 4, 5])
+def test_all_permutations(gpu, rank):
+    # reference test1: dims 2 + r*14/rank, every permutation, 8- and 4-byte elements
+    dim = [2 + r * 14 // rank for r in range(rank)]
+    for perm in itertools.permutations(range(rank)):
+        for es in (8, 4):
+            gpu.check_case(dim, list(perm), es)
+
+
+@pytest.mark.parametrize("rank", [6, 7])
+def test_sampled_permutations(gpu, rank):
+    dim = [2 + r * 14 // rank for r in range(rank)]
+    rng = np.random.default_rng(rank)
+    perms = [list(p) for p in itertools.islice(itertools.permutations(range(rank)), 0, None, 97 if rank == 7 else 17)]
+    perms += [[int(p) for p in rng.permutation(rank)] for _ in range(10)]
+    for perm in perms:
+        for es in (8, 4):
+            gpu.check_case(dim, perm, es)
+
+
+def test_every_candidate_small(gpu):
+    # each candidate of the enumeration is executed, not only the chosen one
+    import cutt_amd as cutt
+    cases = [((43, 67), (1, 0)), ((40, 3, 50, 7), (2, 1, 0, 3)), ((5, 7, 11, 13, 17), (4, 2, 0, 1, 3)),
+             ((31, 549, 2, 3), (3, 0, 2, 1)), ((130, 9, 70), (0, 2, 1)), ((6, 5, 4, 3, 2, 7, 8), (6, 0, 3, 2, 5, 1, 4)),
+             ((3000, 2, 50), (2, 1, 0)), ((70000, 3), (1, 0)), ((3, 70000), (1, 0))]
+    methods = set()
+    for dim, perm in cases:
+        for es in (4, 8):
+            with cutt.Candidates(dim, perm, es) as c:
+                n = len(c)
+            for i in range(n):
+                say("candidate %d/%d dim=%s perm=%s es=%d" % (i, n, dim, perm, es))
+                info = gpu.check_case(dim, list(perm), es, how="candidate", candidate=i)
+                methods.add(info.method_name)
+    assert {"Tiled", "TiledCopy", "Packed", "PackedSplit"} <= methods
+
+
+HAND_PICKED = [  # reference test3, full sizes
+    ((43, 67), (1, 0)),
+    ((65536 * 32, 2), (1, 0)),
+    ((1305, 599, 88), (0, 2, 1)),
+    ((24, 330, 64, 147), (1, 0, 2, 3)),
+    ((2, 5, 9, 12), (0, 1, 2, 3)),
+    ((2, 4, 6, 9, 11, 13), (0, 1, 2, 3, 4, 5)),
+    ((5, 42, 75, 86, 57), (1, 3, 4, 2, 0)),
+    ((5, 3, 2, 9, 14), (0, 1, 3, 2, 4)),
+]
+
+
+@pytest.mark.parametrize("dim,perm", HAND_PICKED)
+def test_hand_picked(gpu, dim, perm):
+    for es in (8, 4):
+        say("hand picked dim=%s perm=%s es=%d" % (dim, perm, es))
+        for how in ("plan", "measure"):
+            info = gpu.check_case(list(dim), list(perm), es, how=how)
+        if list(perm) == sorted(perm):
+            assert info.method_name == "Trivial"
+
+
+def test_forced_methods_large(gpu):
+    # every method on a tensor large enough to need many workgroups
+    import cutt_amd as cutt
+    cases = {
+        cutt.METHOD_TILED: ((1000, 30, 777), (2, 1, 0)),
+        cutt.METHOD_TILEDCOPY: ((1305, 599, 30), (0, 2, 1)),
+        cutt.METHOD_PACKED: ((5, 7, 11, 13, 17, 31), (4, 2, 0, 5, 1, 3)),
+        cutt.METHOD_PACKEDSPLIT: ((200000, 2, 50), (2, 1, 0)),
+    }
+    try:
+        for method, (dim, perm) in cases.items():
+            cutt.set_method_override(method)
+            for es in (8, 4):
+                say("forced %s dim=%s es=%d" % (cutt.METHOD_NAMES[method], dim, es))
+                info = gpu.check_case(list(dim), list(perm), es)
+                assert info.method == method
+    finally:
+        cutt.set_method_override(0)
+
+
+def test_random_ranks_up_to_15(gpu):
+    # reference test2, seeded: random shapes and permutations for ranks 2..15
+    rng = np.random.default_rng(2024)
+    for rank in range(2, 16):
+        for _ in range(4):
+            target = float(rng.uniform(3.0 ** rank, max(3.0 ** rank * 2, 3.0e6)))
+            target = min(target, 2.0e7)
+            dim = [2] * rank
+            while float(np.prod(dim, dtype=np.float64)) < target:
+                dim[int(rng.integers(0, rank))] += 1
+            perm = [int(p) for p in rng.permutation(rank)]
+            es = 8 if rng.random() < 0.5 else 4
+            say("random rank %d dim=%s perm=%s es=%d" % (rank, dim, perm, es))
+            gpu.check_case(dim, perm, es)
+
+
+def test_ten_streams(gpu):
+    # reference test4: ten plans on ten streams executing into the same buffers
+    import torch
+    import cutt_amd as cutt
+    dim, perm = [24, 32, 16, 36, 43, 9], [5, 1, 4, 2, 3, 0]
+    vol = int(np.prod(dim))
+    data = gpu.seeded(vol, 8, 4)
+    d_in = gpu.to_device(data)
+    d_out = torch.full_like(d_in, -1)
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream() for _ in range(10)]
+    handles = []
+    for s in streams:
+        rc, h = cutt.cuttPlan(len(dim), dim, perm, 8, s.cuda_stream)
+        assert rc == cutt.CUTT_SUCCESS
+        assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+        handles.append(h)
+    torch.cuda.synchronize()
+    import oracle
+    assert np.array_equal(gpu.to_host(d_out, 8), oracle.transpose_mt(dim, perm, data, 8))
+    assert len(set(handles)) == 10
+    for h in handles:
+        assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+
+
+def test_error_codes(gpu):
+    # reference src/cutt.cpp:59-82, 193, 287-306
+    import torch
+    import cutt_amd as cutt
+    st = gpu.stream_handle()
+    bad = [((4, 4), (0, 0), 4), ((4, 1), (1, 0), 4), ((4, 4), (1, 0), 2), ((4,), (0,), 4), ((4, 4), (1, 2), 8),
+           ((4, 4), (-1, 0), 8)]
+    for dim, perm, es in bad:
+        rc, _ = cutt.cuttPlan(len(dim), dim, perm, es, st)
+        assert rc == cutt.CUTT_INVALID_PARAMETER
+    a = torch.zeros(16, dtype=torch.int64, device="cuda")
+    b = torch.zeros(16, dtype=torch.int64, device="cuda")
+    rc, _ = cutt.cuttPlanMeasure(2, (4, 4), (1, 0), 8, st, a.data_ptr(), a.data_ptr())
+    assert rc == cutt.CUTT_INVALID_PARAMETER
+    rc, h = cutt.cuttPlan(2, (4, 4), (1, 0), 8, st)
+    assert rc == cutt.CUTT_SUCCESS
+    assert cutt.cuttExecute(h, a.data_ptr(), a.data_ptr()) == cutt.CUTT_INVALID_PARAMETER
+    assert cutt.cuttExecute(h, a.data_ptr(), b.data_ptr()) == cutt.CUTT_SUCCESS
+    torch.cuda.synchronize()
+    assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+    assert cutt.cuttDestroy(h) == cutt.CUTT_INVALID_PLAN
+    assert cutt.cuttExecute(h, a.data_ptr(), b.data_ptr()) == cutt.CUTT_INVALID_PLAN
+    assert cutt.cuttExecute(0xFFFFFFF0, a.data_ptr(), b.data_ptr()) == cutt.CUTT_INVALID_PLAN
+
+
+def test_special_bit_patterns(gpu):
+    # NaNs, infinities, denormals and -0.0 move unchanged (elements are opaque words)
+    words = np.array([0x7FC00001, 0xFFC12345, 0x00000001, 0x80000000, 0x7F800000, 0xFF800000,
+                      0x7FA00000, 0x00000000], dtype=np.uint32)
+    data = np.tile(words, 33 * 65 // 8 + 1)[: 33 * 65]
+    gpu.check_case([33, 65], [1, 0], 4, data=data)
+    data8 = (data.astype(np.uint64) << np.uint64(32)) | np.uint64(0x7FF00000)
+    gpu.check_case([33, 65], [1, 0], 8, data=data8)
