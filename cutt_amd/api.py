@@ -37,6 +37,7 @@ class PlanInfo(ctypes.Structure):
         ("method", ctypes.c_int), ("fromReduced", ctypes.c_int), ("rank", ctypes.c_int),
         ("numMm", ctypes.c_int), ("numMk", ctypes.c_int),
         ("splitRank", ctypes.c_int), ("splitDim", ctypes.c_int), ("numSplit", ctypes.c_int),
+        ("splitRank2", ctypes.c_int), ("splitDim2", ctypes.c_int), ("numSplit2", ctypes.c_int),
         ("volMm", ctypes.c_longlong), ("volMk", ctypes.c_longlong), ("volMmk", ctypes.c_longlong),
         ("volMbar", ctypes.c_longlong), ("volMmkInCont", ctypes.c_longlong),
         ("volMmkOutCont", ctypes.c_longlong), ("volMmkUnsplit", ctypes.c_longlong),

@@ -10,6 +10,7 @@
  * cuttPlanMeasure times each candidate twice and keeps the faster run,
  * because a first launch also pays for loading the kernel.
  */
+#include <algorithm>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
@@ -98,9 +99,12 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.rank = p.pb.rank;
   o.numMm = p.split.numMm;
   o.numMk = p.split.numMk;
-  o.splitRank = p.split.splitRank;
-  o.splitDim = p.split.splitDim;
-  o.numSplit = p.split.numSplit;
+  o.splitRank = p.split.splitRank[0];
+  o.splitDim = p.split.splitDim[0];
+  o.numSplit = p.split.numSplit[0];
+  o.splitRank2 = p.split.splitRank[1];
+  o.splitDim2 = p.split.splitDim[1];
+  o.numSplit2 = p.split.numSplit[1];
   o.volMm = p.split.volMm;
   o.volMk = p.split.volMk;
   o.volMmk = p.split.volMmk;
@@ -145,6 +149,13 @@ bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
   red.set((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType);
   PlannerOptions opt;
   opt.forceMethod = forceMethod;
+  // Tuning knobs for experiments; the defaults are what the library ships with.
+  if (const char* e = std::getenv("CUTT_TILED_ORDER")) opt.tiledOrder = std::atoi(e);
+  if (const char* e = std::getenv("CUTT_XCD_AWARE")) opt.xcdAware = std::atoi(e) != 0;
+  if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
+  if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));
   return createPlans(orig, red, props, opt, plans);
 }
 
@@ -425,7 +436,7 @@ extern "C" int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info) {
 extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                                         long long maxCount) {
   CandidateList* l = (CandidateList*)list;
-  if (!l || index < 0 || index >= (int)l->plans.size() || cls < 0 || cls > 1) return -1;
+  if (!l || index < 0 || index >= (int)l->plans.size() || cls < 0 || cls > 3) return -1;
   const Plan& p = l->plans[index];
   std::vector<long long> v;
   const bool packed = p.method == kPacked || p.method == kPackedSplit;
@@ -442,31 +453,34 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
     case 1:
       if (p.method == kTiled)
         v = {p.tiled.volMm, p.tiled.volMk, p.tiled.strideInK, p.tiled.strideOutM, p.tiled.tilesM,
-             p.tiled.tilesK, p.tiled.volMbar, p.tiled.order};
+             p.tiled.tilesK, p.tiled.volMbar, p.tiled.order, p.tiled.xcdChunk, p.tiled.superM, p.tiled.superK};
       else if (p.method == kTiledCopy)
         v = {p.tcopy.volMm, p.tcopy.volMk, p.tcopy.strideInK, p.tcopy.strideOutK, p.tcopy.tilesM,
-             p.tcopy.tilesK, p.tcopy.volMbar, p.tcopy.order};
+             p.tcopy.tilesK, p.tcopy.volMbar, p.tcopy.order, p.tcopy.xcdChunk, p.tcopy.superM, p.tcopy.superK};
       else
         return -1;
       break;
     case 2:
       if (!packed) return -1;
-      v = {p.packed.numThreads, p.packed.volMbar, p.packed.numSplit, p.packed.slabFloor,
-           p.packed.slabRem, p.packed.splitStrideIn, p.packed.splitStrideOut, p.packed.itemsPerBlock,
-           p.packed.padShift, p.packed.ldsElems};
+      v = {p.packed.numThreads, p.packed.volMbar, p.packed.itemsPerBlock, p.packed.padShift,
+           p.packed.ldsElems, p.packed.xcdChunk, p.packed.elemsPerThread};
+      for (int i = 0; i < 2; i++) {
+        const cuttHipSplitRank& sr = p.packed.split[i];
+        v.insert(v.end(), {sr.numSplit, sr.slabFloor, sr.slabRem, sr.strideIn, sr.strideOut});
+      }
       break;
     case 3: {
       if (!packed) return -1;
       const cuttHipPackedClass& k = p.packed.cls[cls];
-      v = {k.vol, k.inCont, k.outCont, k.inMagic, k.outMagic, k.nRowsIn, k.nRowsOut};
+      v = {k.vol, k.inCont, k.outCont};
     } break;
     case 4:
       if (!packed) return -1;
-      v.assign(p.tab[cls].rowIn.begin(), p.tab[cls].rowIn.end());
+      v.assign(p.tab[cls].inOff.begin(), p.tab[cls].inOff.end());
       break;
     case 5:
       if (!packed) return -1;
-      v.assign(p.tab[cls].rowOut.begin(), p.tab[cls].rowOut.end());
+      v.assign(p.tab[cls].outOff.begin(), p.tab[cls].outOff.end());
       break;
     case 6:
       if (!packed) return -1;

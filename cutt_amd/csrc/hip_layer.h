@@ -74,7 +74,12 @@ typedef struct cuttHipTiledArgs {
   uint32_t strideOutM;
   int tilesM, tilesK; /* ceil(volMm/64), ceil(volMk/64) */
   int volMbar;
-  int order;          /* workgroup-index decoding: 0 = Mbar fastest, 1 = tiles along Mm fastest, 2 = tiles along Mk fastest */
+  int order;          /* logical numbering of the workgroups: 0 = Mbar fastest, 1 = tiles along Mm
+                         fastest, 2 = tiles along Mk fastest, 3 / 4 = superM x superK super-tiles with the
+                         tiles along Mm / along Mk running fastest inside and between them */
+  uint32_t xcdChunk;  /* 0: workgroup b is logical position b; else (b % 8)*xcdChunk + b/8, and the
+                         grid has 8*xcdChunk workgroups */
+  uint32_t superM, superK;
   cuttHipMbar mbar;
 } cuttHipTiledArgs;
 
@@ -91,49 +96,57 @@ typedef struct cuttHipTiledCopyArgs {
   int tilesM, tilesK;
   int volMbar;
   int order;
+  uint32_t xcdChunk;
+  uint32_t superM, superK;
   cuttHipMbar mbar;
 } cuttHipTiledCopyArgs;
 
 /*
- * Index tables of a Packed / PackedSplit plan for one slab size (device
- * pointers).  The staged block holds `vol` elements.  In input-compact order
- * element p lies in row p / inCont at column p % inCont, and is read from
- * input offset rowIn[row] + column; it is stored in LDS slot
- * p + (p >> padShift).  In output-compact order element q is written to
- * output offset rowOut[q / outCont] + q % outCont and taken from LDS slot
- * shIdx[q] (padding included).  inMagic/outMagic = ceil(2^32 / inCont|outCont)
- * for the multiply-high division.
+ * Index-remap tables of a Packed / PackedSplit plan for one slab-size class (device pointers,
+ * `vol` entries each).  The staged block holds `vol` elements.  Element p in input-compact
+ * order is read from input offset inOff[p] and parked in LDS slot p + (p >> padShift).
+ * Element q in output-compact order is written to output offset outOff[q] and taken from LDS
+ * slot shIdx[q] (padding included).  A workgroup reads its slice of the tables once and keeps
+ * it in registers for all the work items it handles.
  */
 typedef struct cuttHipPackedClass {
   int vol;
-  int inCont, outCont;
-  uint32_t inMagic, outMagic;
-  int nRowsIn, nRowsOut;
-  const uint32_t* rowIn;
-  const uint32_t* rowOut;
+  int inCont, outCont;       /* contiguous run lengths (informational) */
+  const uint32_t* inOff;
+  const uint32_t* outOff;
   const uint16_t* shIdx;
 } cuttHipPackedClass;
 
+/* One split rank of a PackedSplit plan: the rank is cut into numSplit slabs; slab s covers
+ * [s*slabFloor + min(s, slabRem), ...) and has slabFloor + (s < slabRem) entries.  An unused
+ * slot has numSplit 1, slabRem 0 and zero strides. */
+typedef struct cuttHipSplitRank {
+  int numSplit;
+  int slabFloor, slabRem;
+  uint32_t strideIn, strideOut; /* global strides of the rank */
+} cuttHipSplitRank;
+
 /*
- * Packed and PackedSplit methods.  Work items are (Mbar position m, slab s),
- * numbered w = m*numSplit + s; workgroup b handles items
- * [b*itemsPerBlock, (b+1)*itemsPerBlock).  Slab s covers
- * [s*slabFloor + min(s, slabRem), ...) of the split rank and has
- * slabFloor + (s < slabRem) entries: class 1 if s < slabRem, else class 0.
- * Packed is the case numSplit == 1 (one slab of class 0, no split rank).
+ * Packed and PackedSplit methods.  A staged block is the index set Mmk with up to two of its
+ * ranks cut into slabs (typically the last rank of the input-contiguous set and the last rank of
+ * the output-contiguous set, which makes the block a 2-D tile over fused rank sets).  Work items
+ * are (Mbar position m, slab s1, slab s0), numbered w = (m*numSplit1 + s1)*numSplit0 + s0;
+ * workgroup b handles items [b*itemsPerBlock, (b+1)*itemsPerBlock).  The slab sizes select the
+ * table class: cls[(s0 < slabRem0) + 2*(s1 < slabRem1)].  Packed is the case without split ranks.
  */
 typedef struct cuttHipPackedArgs {
   int elemSize;
   int numThreads;
   int volMbar;
-  int numSplit;
-  int slabFloor, slabRem;
-  uint32_t splitStrideIn, splitStrideOut; /* global strides of the split rank */
+  cuttHipSplitRank split[2];
   int itemsPerBlock;
+  int elemsPerThread;  /* 1, 2, 4 or 8: numThreads*elemsPerThread >= vol of every class */
   int padShift;        /* LDS slot(p) = p + (p >> padShift); 31 = no padding */
   int ldsElems;        /* element slots in the LDS data buffer (padding included) */
-  int maxRowsIn, maxRowsOut, maxVol; /* maxima over the classes: LDS table sizes */
-  cuttHipPackedClass cls[2];
+  int maxVol;          /* largest class volume */
+  uint32_t xcdChunk;   /* 0: workgroup b is logical block b; else logical block = (b % 8)*xcdChunk + b/8
+                          and the grid has 8*xcdChunk workgroups */
+  cuttHipPackedClass cls[4];
   cuttHipMbar mbar;
 } cuttHipPackedArgs;
 

@@ -13,11 +13,13 @@
  *    and read from the kernel-argument segment (scalar loads), instead of
  *    one-table-entry-per-lane plus cross-lane shuffles;
  *  - Tiled stages a 64x64 tile in LDS padded to 65 columns (conflict-free for
- *    both 4- and 8-byte words); each lane keeps 16 loads in flight;
- *  - Packed/PackedSplit keep their index-remap tables in LDS: a u16 gather
- *    index per element plus one offset per contiguous row, with the
- *    row/column split done by a multiply-high; the LDS data buffer is skewed
- *    by one slot per 2^padShift to break power-of-two bank strides;
+ *    both 4- and 8-byte words); each lane keeps 16 loads in flight; edges are handled by
+ *    clamping indices, not by branches, so the memory instructions stay back to back;
+ *  - Packed/PackedSplit take their index remap from tables the planner precomputed in device
+ *    memory (input offset, output offset and LDS gather slot per staged element); a workgroup
+ *    loads its slice once and keeps it in registers while it loops over its work items, so the
+ *    loop body is load, LDS write, LDS read, store; the LDS buffer is skewed by one slot per
+ *    2^padShift to break power-of-two bank strides;
  *  - workgroups are short-lived and small (a tile, or a few Mbar positions),
  *    thousands are in flight: on this chip that streams faster than a
  *    persistent grid-stride loop.
@@ -52,25 +54,60 @@ __device__ __forceinline__ void mbarOffsets(const cuttHipMbar& mb, uint32_t m, u
   offOut = oo;
 }
 
-// Workgroup index -> (tile along Mm, tile along Mk, Mbar position).
-__device__ __forceinline__ void decodeTile(uint32_t bid, int order, uint32_t tilesM, uint32_t tilesK,
-                                           uint32_t volMbar, uint32_t& tm, uint32_t& tk, uint32_t& m) {
-  if (order == 0) {
-    const uint32_t t = bid / volMbar;
-    m = bid - t * volMbar;
+// Workgroup index -> (tile along Mm, tile along Mk, Mbar position).  Returns false for the
+// padding workgroups of order 3.
+//
+// The chip has 8 XCDs with private L2s and hands workgroup b to XCD b % 8, so neighbouring
+// tiles - which share the 128-byte lines at their unaligned edges - would otherwise always land
+// in different L2s.  With xcdChunk != 0, XCD x walks its own contiguous chunk of the logical
+// sequence.  Orders 0-2 number the logical sequence with the Mbar position, the tile along Mm or
+// the tile along Mk running fastest; orders 3 and 4 visit the tiles in superM x superK super-tiles, so
+// that both the read neighbours (along Mm) and the write neighbours (along Mk) of a tile are
+// resident in the same L2 at about the same time.
+constexpr uint32_t kNumXcd = 8;
+
+struct TileOrder {
+  int order;
+  uint32_t xcdChunk, superM, superK;
+};
+
+__device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint32_t tilesM,
+                                           uint32_t tilesK, uint32_t volMbar, uint32_t& tm,
+                                           uint32_t& tk, uint32_t& m) {
+  const uint32_t l = o.xcdChunk ? (bid % kNumXcd) * o.xcdChunk + bid / kNumXcd : bid;
+  if (o.order == 0) {
+    const uint32_t t = l / volMbar;
+    m = l - t * volMbar;
     tk = t / tilesM;
     tm = t - tk * tilesM;
-  } else if (order == 1) {
-    const uint32_t t = bid / tilesM;
-    tm = bid - t * tilesM;
+    return tk < tilesK;
+  } else if (o.order == 1) {
+    const uint32_t t = l / tilesM;
+    tm = l - t * tilesM;
     m = t / tilesK;
     tk = t - m * tilesK;
-  } else {
-    const uint32_t t = bid / tilesK;
-    tk = bid - t * tilesK;
+    return m < volMbar;
+  } else if (o.order == 2) {
+    const uint32_t t = l / tilesK;
+    tk = l - t * tilesK;
     m = t / tilesM;
     tm = t - m * tilesM;
+    return m < volMbar;
   }
+  const uint32_t nSuperM = (tilesM + o.superM - 1) / o.superM, nSuperK = (tilesK + o.superK - 1) / o.superK;
+  const uint32_t per = o.superM * o.superK;
+  const uint32_t w = l % per;
+  const uint32_t t = l / per;
+  const uint32_t st = t % (nSuperM * nSuperK);
+  m = t / (nSuperM * nSuperK);
+  if (o.order == 3) {  // inside a super-tile the tiles along Mm run fastest
+    tm = (st % nSuperM) * o.superM + (w % o.superM);
+    tk = (st / nSuperM) * o.superK + (w / o.superM);
+  } else {             // order 4: the tiles along Mk run fastest, super-tiles advance along Mk first
+    tk = (st % nSuperK) * o.superK + (w % o.superK);
+    tm = (st / nSuperK) * o.superM + (w / o.superK);
+  }
+  return m < volMbar && tm < tilesM && tk < tilesK;
 }
 
 // ---------------------------------------------------------------------------
@@ -83,7 +120,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
   __shared__ T tile[kTile][kTile + 1];
 
   uint32_t tm, tk, m;
-  decodeTile(blockIdx.x, a.order, a.tilesM, a.tilesK, a.volMbar, tm, tk, m);
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(a.mbar, m, offIn, offOut);
 
@@ -92,33 +129,43 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
   const uint32_t m0 = tm * kTile, k0 = tk * kTile;
   const uint32_t volMm = a.volMm, volMk = a.volMk;
 
+  // Edge tiles are handled without branches: indices are clamped to the last valid row / column,
+  // so out-of-range lanes repeat the access of the edge element (same address, same value).  That
+  // keeps the loop bodies straight-line code, and all 16 loads of a lane go out back to back.
+  const uint32_t wM = min((uint32_t)kTile, volMm - m0) - 1;  // last valid column / row inside the tile
+  const uint32_t wK = min((uint32_t)kTile, volMk - k0) - 1;
+
   // Read: lanes run along input rank 0, rows along the Mk rank.
   {
-    const uint32_t x = m0 + lane;
-    const bool xok = x < volMm;
+    const uint32_t cx = min(lane, wM);
+    const T* src = in + (offIn + m0 + cx);
     T v[kTileRows];
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = wave + kWaves * j;
-      const uint32_t k = k0 + r;
-      if (xok && k < volMk) v[j] = in[offIn + x + k * a.strideInK];
+      const uint32_t r = min(wave + kWaves * j, wK);
+      v[j] = src[(k0 + r) * a.strideInK];
     }
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = wave + kWaves * j;
-      if (xok && k0 + r < volMk) tile[r][lane] = v[j];
+      const uint32_t r = min(wave + kWaves * j, wK);
+      tile[r][cx] = v[j];
     }
   }
   __syncthreads();
   // Write: lanes run along the Mk rank (contiguous in the output).
   {
-    const uint32_t k = k0 + lane;
-    const bool kok = k < volMk;
+    const uint32_t ck = min(lane, wK);
+    T* dst = out + (offOut + k0 + ck);
+    T v[kTileRows];
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = wave + kWaves * j;
-      const uint32_t x = m0 + r;
-      if (kok && x < volMm) out[offOut + k + x * a.strideOutM] = tile[lane][r];
+      const uint32_t r = min(wave + kWaves * j, wM);
+      v[j] = tile[ck][r];
+    }
+#pragma unroll
+    for (int j = 0; j < kTileRows; j++) {
+      const uint32_t r = min(wave + kWaves * j, wM);
+      dst[(m0 + r) * a.strideOutM] = v[j];
     }
   }
 }
@@ -131,125 +178,110 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
                                                                 const T* __restrict__ in,
                                                                 T* __restrict__ out) {
   uint32_t tm, tk, m;
-  decodeTile(blockIdx.x, a.order, a.tilesM, a.tilesK, a.volMbar, tm, tk, m);
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(a.mbar, m, offIn, offOut);
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
-  const uint32_t x = tm * kTile + lane;
-  const uint32_t k0 = tk * kTile;
-  const bool xok = x < (uint32_t)a.volMm;
-  const uint32_t volMk = a.volMk;
+  const uint32_t m0 = tm * kTile, k0 = tk * kTile;
+  // Clamped indices instead of branches, as in the tiled kernel.
+  const uint32_t cx = min(lane, min((uint32_t)kTile, (uint32_t)a.volMm - m0) - 1);
+  const uint32_t wK = min((uint32_t)kTile, (uint32_t)a.volMk - k0) - 1;
+  const T* src = in + (offIn + m0 + cx);
+  T* dst = out + (offOut + m0 + cx);
 
   T v[kTileRows];
 #pragma unroll
   for (int j = 0; j < kTileRows; j++) {
-    const uint32_t k = k0 + wave + kWaves * j;
-    if (xok && k < volMk) v[j] = in[offIn + x + k * a.strideInK];
+    const uint32_t r = min(wave + kWaves * j, wK);
+    v[j] = src[(k0 + r) * a.strideInK];
   }
 #pragma unroll
   for (int j = 0; j < kTileRows; j++) {
-    const uint32_t k = k0 + wave + kWaves * j;
-    if (xok && k < volMk) out[offOut + x + k * a.strideOutK] = v[j];
+    const uint32_t r = min(wave + kWaves * j, wK);
+    dst[(k0 + r) * a.strideOutK] = v[j];
   }
 }
 
 // ---------------------------------------------------------------------------
 // Packed / PackedSplit: stage a block of Mmk through LDS with remap tables.
 // ---------------------------------------------------------------------------
-constexpr int kPackedUnroll = 4;
 
-// n / d for n < 2^16, 2 <= d <= 2^16 with magic = ceil(2^32 / d); d == 1 handled apart.
-__device__ __forceinline__ uint32_t divSmall(uint32_t n, uint32_t d, uint32_t magic) {
-  return d == 1 ? n : __umulhi(n, magic);
-}
-
-template <typename T>
-__global__ void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
+// E = elements per lane.  Every lane keeps its E table entries in registers, so that the loop
+// over work items does no index arithmetic beyond adding the item's base offsets.
+template <typename T, int E>
+__global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
                              T* __restrict__ out) {
   extern __shared__ __align__(16) unsigned char ldsRaw[];
   T* buf = reinterpret_cast<T*>(ldsRaw);
-  uint32_t* sRowIn = reinterpret_cast<uint32_t*>(buf + a.ldsElems);
-  uint32_t* sRowOut = sRowIn + a.maxRowsIn;
-  uint16_t* sSh = reinterpret_cast<uint16_t*>(sRowOut + a.maxRowsOut);
 
   const uint32_t tid = threadIdx.x;
   const uint32_t nt = blockDim.x;
-  const uint32_t numSplit = a.numSplit;
-  const uint32_t totalItems = (uint32_t)a.volMbar * numSplit;
-  const uint32_t w0 = blockIdx.x * (uint32_t)a.itemsPerBlock;
+  const uint32_t ns0 = a.split[0].numSplit, ns1 = a.split[1].numSplit;
+  const uint32_t totalItems = (uint32_t)a.volMbar * ns0 * ns1;
+  // XCD-aware numbering: XCD x (= blockIdx.x % 8) walks its own contiguous chunk of the work
+  // items, so that neighbouring slabs and Mbar positions share an L2.
+  uint32_t lb = blockIdx.x;
+  if (a.xcdChunk) lb = (blockIdx.x % kNumXcd) * (uint32_t)a.xcdChunk + blockIdx.x / kNumXcd;
+  const uint32_t w0 = lb * (uint32_t)a.itemsPerBlock;
   const uint32_t w1 = min(w0 + (uint32_t)a.itemsPerBlock, totalItems);
-  const uint32_t slabRem = a.slabRem;
+  const uint32_t rem0 = a.split[0].slabRem, rem1 = a.split[1].slabRem;
   const int padShift = a.padShift;
 
+  // Lanes whose element index lies beyond the block repeat the block's last element (same
+  // addresses, same value), so that the code below has no branches and every lane's E loads go
+  // out back to back.
+  uint32_t inOff[E], outOff[E], shSlot[E], ldsSlot[E];
   int loaded = -1;
   for (uint32_t w = w0; w < w1; w++) {
-    const uint32_t m = w / numSplit;
-    const uint32_t s = w - m * numSplit;
-    const int c = (s < slabRem) ? 1 : 0;
-    const uint32_t p0 = s * (uint32_t)a.slabFloor + min(s, slabRem);
+    const uint32_t t = w / ns0;
+    const uint32_t s0 = w - t * ns0;
+    const uint32_t m = t / ns1;
+    const uint32_t s1 = t - m * ns1;
+    const int c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
+    const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
+    const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
 
     uint32_t offIn, offOut;
     mbarOffsets(a.mbar, m, offIn, offOut);
-    offIn += p0 * a.splitStrideIn;
-    offOut += p0 * a.splitStrideOut;
+    offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
+    offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
 
-    const uint32_t vol = a.cls[c].vol;
-    const uint32_t inCont = a.cls[c].inCont, outCont = a.cls[c].outCont;
-    const uint32_t inMagic = a.cls[c].inMagic, outMagic = a.cls[c].outMagic;
-
-    __syncthreads();  // the previous item has finished reading the LDS buffer
-    if (c != loaded) {
-      const uint32_t nIn = a.cls[c].nRowsIn, nOut = a.cls[c].nRowsOut;
-      const uint32_t* gIn = a.cls[c].rowIn;
-      const uint32_t* gOut = a.cls[c].rowOut;
+    if (c != loaded) {  // wave-uniform: the class changes at most a few times per workgroup
+      const uint32_t last = (uint32_t)a.cls[c].vol - 1;
+      const uint32_t* gIn = a.cls[c].inOff;
+      const uint32_t* gOut = a.cls[c].outOff;
       const uint16_t* gSh = a.cls[c].shIdx;
-      for (uint32_t i = tid; i < nIn; i += nt) sRowIn[i] = gIn[i];
-      for (uint32_t i = tid; i < nOut; i += nt) sRowOut[i] = gOut[i];
-      for (uint32_t i = tid; i < vol; i += nt) sSh[i] = gSh[i];
+#pragma unroll
+      for (int j = 0; j < E; j++) {
+        const uint32_t p = min(tid + j * nt, last);
+        inOff[j] = gIn[p];
+        outOff[j] = gOut[p];
+        shSlot[j] = gSh[p];
+        ldsSlot[j] = p + (p >> padShift);
+      }
       loaded = c;
-      __syncthreads();
     }
+    const T* src = in + offIn;
+    T* dst = out + offOut;
 
-    // Global -> LDS in input-compact order.
-    for (uint32_t base = tid; base < vol; base += nt * kPackedUnroll) {
-      T v[kPackedUnroll];
+    T v[E];
 #pragma unroll
-      for (int u = 0; u < kPackedUnroll; u++) {
-        const uint32_t p = base + u * nt;
-        if (p < vol) {
-          const uint32_t row = divSmall(p, inCont, inMagic);
-          const uint32_t col = p - row * inCont;
-          v[u] = in[offIn + sRowIn[row] + col];
-        }
-      }
+    for (int j = 0; j < E; j++) v[j] = src[inOff[j]];
+    __syncthreads();  // the previous item has finished reading the LDS buffer
 #pragma unroll
-      for (int u = 0; u < kPackedUnroll; u++) {
-        const uint32_t p = base + u * nt;
-        if (p < vol) buf[p + (p >> padShift)] = v[u];
-      }
-    }
+    for (int j = 0; j < E; j++) buf[ldsSlot[j]] = v[j];
     __syncthreads();
-    // LDS -> global in output-compact order.
-    for (uint32_t base = tid; base < vol; base += nt * kPackedUnroll) {
 #pragma unroll
-      for (int u = 0; u < kPackedUnroll; u++) {
-        const uint32_t q = base + u * nt;
-        if (q < vol) {
-          const uint32_t row = divSmall(q, outCont, outMagic);
-          const uint32_t col = q - row * outCont;
-          out[offOut + sRowOut[row] + col] = buf[sSh[q]];
-        }
-      }
-    }
+    for (int j = 0; j < E; j++) v[j] = buf[shSlot[j]];
+#pragma unroll
+    for (int j = 0; j < E; j++) dst[outOff[j]] = v[j];
   }
 }
 
 size_t packedLdsBytes(const cuttHipPackedArgs* a) {
-  size_t b = (size_t)a->ldsElems * a->elemSize;
-  b += sizeof(uint32_t) * ((size_t)a->maxRowsIn + a->maxRowsOut);
-  b += sizeof(uint16_t) * (size_t)a->maxVol;
+  const size_t b = (size_t)a->ldsElems * a->elemSize;
   return (b + 15) & ~(size_t)15;
 }
 
@@ -258,6 +290,23 @@ bool mbarOk(const cuttHipMbar& mb) {
   for (int k = 0; k < mb.n; k++)
     if (mb.d[k].extent == 0) return false;
   return true;
+}
+
+// Number of workgroups of a tiled launch; checks the ordering parameters.
+bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk, uint32_t superM,
+              uint32_t superK, uint64_t& blocks) {
+  uint64_t logical = (uint64_t)tilesM * tilesK * (uint64_t)volMbar;
+  if (order >= 3) {
+    if (superM < 1 || superK < 1) return false;
+    logical = (uint64_t)((tilesM + superM - 1) / superM) * ((tilesK + superK - 1) / superK) * superM * superK *
+              (uint64_t)volMbar;
+  }
+  blocks = logical;
+  if (xcdChunk) {
+    if ((uint64_t)xcdChunk * kNumXcd < logical) return false;
+    blocks = (uint64_t)xcdChunk * kNumXcd;
+  }
+  return blocks > 0 && blocks <= 0x7fffffffull;
 }
 
 // Allow dynamic LDS up to the device limit for a kernel (once per process and kernel).
@@ -275,10 +324,11 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 2 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 4 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
-  const uint64_t blocks = (uint64_t)a->tilesM * a->tilesK * (uint64_t)a->volMbar;
-  if (blocks == 0 || blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
+  uint64_t blocks = 0;
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+    return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   if (a->elemSize == 4)
     hipLaunchKernelGGL(tiledKernel<uint32_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
@@ -294,10 +344,11 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 2 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 4 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
-  const uint64_t blocks = (uint64_t)a->tilesM * a->tilesK * (uint64_t)a->volMbar;
-  if (blocks == 0 || blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
+  uint64_t blocks = 0;
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+    return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   if (a->elemSize == 4)
     hipLaunchKernelGGL(tiledCopyKernel<uint32_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
@@ -311,43 +362,71 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
 extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, void* out, void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
-      (a->numThreads & 63) || a->volMbar < 1 || a->numSplit < 1 || a->itemsPerBlock < 1 ||
-      a->slabRem < 0 || a->slabRem >= a->numSplit || a->padShift < 1 || a->padShift > 31 ||
-      a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar))
+      (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
+      (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
+       a->elemsPerThread != 8) ||
+      a->padShift > 31 || a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
-  const int ncls = (a->slabRem > 0) ? 2 : 1;
-  for (int c = 0; c < ncls; c++) {
+  uint64_t items = (uint64_t)a->volMbar;
+  for (int i = 0; i < 2; i++) {
+    const cuttHipSplitRank& sr = a->split[i];
+    if (sr.numSplit < 1 || sr.slabRem < 0 || sr.slabRem >= sr.numSplit || sr.slabFloor < 0)
+      return (int)hipErrorInvalidValue;
+    items *= (uint64_t)sr.numSplit;
+    if (items > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
+  }
+  for (int c = 0; c < 4; c++) {
+    // class c is used only if the split ranks it refers to have slabs of the larger size
+    if (((c & 1) && a->split[0].slabRem == 0) || ((c & 2) && a->split[1].slabRem == 0)) continue;
     const cuttHipPackedClass& k = a->cls[c];
-    if (k.vol < 1 || k.vol > a->maxVol || k.inCont < 1 || k.outCont < 1 || k.nRowsIn > a->maxRowsIn ||
-        k.nRowsOut > a->maxRowsOut || (int64_t)k.nRowsIn * k.inCont != k.vol ||
-        (int64_t)k.nRowsOut * k.outCont != k.vol || !k.rowIn || !k.rowOut || !k.shIdx)
+    if (k.vol < 1 || k.vol > a->maxVol || (int64_t)a->numThreads * a->elemsPerThread < k.vol || !k.inOff ||
+        !k.outOff || !k.shIdx)
       return (int)hipErrorInvalidValue;
     const uint32_t last = (uint32_t)k.vol - 1;
     if ((int)(last + (last >> a->padShift)) >= a->ldsElems) return (int)hipErrorInvalidValue;
   }
-  const uint64_t items = (uint64_t)a->volMbar * a->numSplit;
-  const uint64_t blocks = (items + a->itemsPerBlock - 1) / a->itemsPerBlock;
-  if (items > 0x7fffffffull || blocks == 0) return (int)hipErrorInvalidConfiguration;
+  uint64_t blocks = (items + a->itemsPerBlock - 1) / a->itemsPerBlock;
+  if (blocks == 0) return (int)hipErrorInvalidConfiguration;
+  if (a->xcdChunk) {
+    if ((uint64_t)a->xcdChunk * kNumXcd < blocks) return (int)hipErrorInvalidValue;
+    blocks = (uint64_t)a->xcdChunk * kNumXcd;
+    if (blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
+  }
   const size_t lds = packedLdsBytes(a);
 
-  static bool ldsOptIn = false;  // benign if two threads race: the call is idempotent
+  static bool ldsOptIn = false;  // benign if two threads race: the calls are idempotent
   if (!ldsOptIn) {
     int dev = 0;
     hipDeviceProp_t prop;
     hipError_t e = hipGetDevice(&dev);
     if (e == hipSuccess) e = hipGetDeviceProperties(&prop, dev);
     if (e != hipSuccess) return (int)e;
-    int r = allowLargeLds(packedKernel<uint32_t>, prop.sharedMemPerBlock);
-    if (r == 0) r = allowLargeLds(packedKernel<uint64_t>, prop.sharedMemPerBlock);
+    const size_t m = prop.sharedMemPerBlock;
+    int r = 0;
+#define CUTT_ALLOW(T, E) if (r == 0) r = allowLargeLds(packedKernel<T, E>, m)
+    CUTT_ALLOW(uint32_t, 1); CUTT_ALLOW(uint32_t, 2); CUTT_ALLOW(uint32_t, 4); CUTT_ALLOW(uint32_t, 8);
+    CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
+#undef CUTT_ALLOW
     if (r != 0) return r;
     ldsOptIn = true;
   }
   hipStream_t s = (hipStream_t)stream;
-  if (a->elemSize == 4)
-    hipLaunchKernelGGL(packedKernel<uint32_t>, dim3((uint32_t)blocks), dim3(a->numThreads), lds, s, *a,
-                       (const uint32_t*)in, (uint32_t*)out);
-  else
-    hipLaunchKernelGGL(packedKernel<uint64_t>, dim3((uint32_t)blocks), dim3(a->numThreads), lds, s, *a,
-                       (const uint64_t*)in, (uint64_t*)out);
+  const dim3 grid((uint32_t)blocks), block(a->numThreads);
+#define CUTT_LAUNCH_PACKED(T, E) \
+  hipLaunchKernelGGL((packedKernel<T, E>), grid, block, lds, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_PACKED_E(T)                        \
+  switch (a->elemsPerThread) {                         \
+    case 1: CUTT_LAUNCH_PACKED(T, 1); break;           \
+    case 2: CUTT_LAUNCH_PACKED(T, 2); break;           \
+    case 4: CUTT_LAUNCH_PACKED(T, 4); break;           \
+    default: CUTT_LAUNCH_PACKED(T, 8); break;          \
+  }
+  if (a->elemSize == 4) {
+    CUTT_LAUNCH_PACKED_E(uint32_t)
+  } else {
+    CUTT_LAUNCH_PACKED_E(uint64_t)
+  }
+#undef CUTT_LAUNCH_PACKED_E
+#undef CUTT_LAUNCH_PACKED
   return (int)hipGetLastError();
 }

@@ -259,22 +259,24 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   } else {
     if (!plan.buildTables()) return false;
     const cuttHipPackedArgs& a = plan.packed;
-    const uint32_t items = (uint32_t)a.volMbar * (uint32_t)a.numSplit;
+    const uint32_t ns0 = (uint32_t)a.split[0].numSplit, ns1 = (uint32_t)a.split[1].numSplit;
+    const uint32_t items = (uint32_t)a.volMbar * ns0 * ns1;
     const int ns = (numSamples == 0 || (uint32_t)numSamples > items) ? (int)items : numSamples;
     std::uniform_int_distribution<uint32_t> pick(0, items - 1);
     for (int i = 0; i < ns; i++) {
       const uint32_t w = ((uint32_t)ns == items) ? (uint32_t)i : pick(rng);
-      const uint32_t m = w / a.numSplit, s = w % a.numSplit;
-      const int cls = s < (uint32_t)a.slabRem ? 1 : 0;
-      const int64_t p0 = (int64_t)s * a.slabFloor + std::min<int64_t>(s, a.slabRem);
+      const uint32_t s0 = w % ns0, t = w / ns0, s1 = t % ns1, m = t / ns1;
+      const int cls = (s0 < (uint32_t)a.split[0].slabRem ? 1 : 0) + (s1 < (uint32_t)a.split[1].slabRem ? 2 : 0);
+      const int64_t p0 = (int64_t)s0 * a.split[0].slabFloor + std::min<int64_t>(s0, a.split[0].slabRem);
+      const int64_t p1 = (int64_t)s1 * a.split[1].slabFloor + std::min<int64_t>(s1, a.split[1].slabRem);
       int64_t offIn, offOut;
       mbarOffsets(a.mbar, m, offIn, offOut);
-      offIn += p0 * a.splitStrideIn;
-      offOut += p0 * a.splitStrideOut;
+      offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
+      offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
       total.add(packedSample(plan, cls, offIn, offOut), (double)items / ns);
     }
     // Every workgroup loads its tables once from L2.
-    tableBytes = (double)plan.numBlocks * (2.0 * a.maxVol + 4.0 * (a.maxRowsIn + a.maxRowsOut));
+    tableBytes = (double)plan.numBlocks * 10.0 * a.maxVol;
   }
   r.rdLines = total.rdLines; r.wrLines = total.wrLines;
   r.rdInstr = total.rdInstr; r.wrInstr = total.wrInstr;

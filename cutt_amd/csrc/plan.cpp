@@ -10,6 +10,7 @@
 #include "plan.h"
 
 #include <algorithm>
+#include <cmath>
 #include <cstdio>
 #include <cstring>
 #include <sstream>
@@ -20,6 +21,7 @@ namespace {
 constexpr int kTile = 64;
 constexpr int kPadShift = 5;            // one LDS pad slot per 32 elements
 constexpr int64_t kMaxLdsSlots = 65536; // the gather index is 16 bits wide
+constexpr int64_t kNumXcd = 8;          // XCDs (private L2s); workgroup b runs on XCD b % 8
 
 inline int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int roundUp64(int64_t v) { return (int)(ceilDiv(v, 64) * 64); }
@@ -133,17 +135,16 @@ void Split::update(int numMm_, int numMk_, const Problem& pb) {
   }
   sizeMbar = rank - sizeMmk;
   volMbar = pb.volume / volMmk;
-  if (splitRank >= 0) {
-    splitDim = pb.dim[splitRank];
-    volMmkUnsplit = volMmk / splitDim;
-  } else {
-    splitDim = 0;
-    volMmkUnsplit = volMmk;
+  volMmkUnsplit = volMmk;
+  for (int i = 0; i < 2; i++) {
+    splitDim[i] = splitRank[i] >= 0 ? pb.dim[splitRank[i]] : 0;
+    if (splitRank[i] >= 0) volMmkUnsplit /= splitDim[i];
   }
   volMmkInCont = 1;
   for (int r = 0; r < rank && inMmk[r]; r++) {
-    if (r == splitRank) {
-      volMmkInCont *= slabMax();
+    const int slot = splitSlot(r);
+    if (slot >= 0) {
+      volMmkInCont *= slabMax(slot);
       break;
     }
     volMmkInCont *= pb.dim[r];
@@ -151,8 +152,9 @@ void Split::update(int numMm_, int numMk_, const Problem& pb) {
   volMmkOutCont = 1;
   for (int j = 0; j < rank && inMmk[pb.perm[j]]; j++) {
     const int r = pb.perm[j];
-    if (r == splitRank) {
-      volMmkOutCont *= slabMax();
+    const int slot = splitSlot(r);
+    if (slot >= 0) {
+      volMmkOutCont *= slabMax(slot);
       break;
     }
     volMmkOutCont *= pb.dim[r];
@@ -162,7 +164,7 @@ void Split::update(int numMm_, int numMk_, const Problem& pb) {
 int64_t Split::volStaged() const {
   switch (method) {
     case kPacked: return volMmk;
-    case kPackedSplit: return (int64_t)slabMax() * volMmkUnsplit;
+    case kPackedSplit: return (int64_t)slabMax(0) * slabMax(1) * volMmkUnsplit;
     case kTiled: return kTile * kTile;
     default: return 0;
   }
@@ -194,8 +196,7 @@ Plan& Plan::operator=(Plan&& o) noexcept {
   ldsBytes = o.ldsBytes;
   numBlocks = o.numBlocks;
   numThreads = o.numThreads;
-  tab[0] = std::move(o.tab[0]);
-  tab[1] = std::move(o.tab[1]);
+  for (int c = 0; c < 4; c++) tab[c] = std::move(o.tab[c]);
   tablesBuilt = o.tablesBuilt;
   dTables = o.dTables;
   o.dTables = nullptr;
@@ -207,9 +208,9 @@ void Plan::release() {
   if (dTables) {
     cuttHipFree(dTables);
     dTables = nullptr;
-    for (int c = 0; c < 2; c++) {
-      packed.cls[c].rowIn = nullptr;
-      packed.cls[c].rowOut = nullptr;
+    for (int c = 0; c < 4; c++) {
+      packed.cls[c].inOff = nullptr;
+      packed.cls[c].outOff = nullptr;
       packed.cls[c].shIdx = nullptr;
     }
   }
@@ -240,10 +241,15 @@ void enumerateOffsets(const std::vector<RadixDim>& dims, int64_t count, std::vec
   }
 }
 
-void fillMbar(const Problem& pb, const std::vector<char>& inMmk, cuttHipMbar& mb) {
+// Mbar table.  The order of its ranks is the order in which consecutive workgroups walk the
+// remaining index space: mbarOrder 0 = input order (consecutive workgroups read neighbouring
+// memory), 1 = output order (they write neighbouring memory, so the partly written 128-byte
+// lines at the ends of their runs meet in the same L2).
+void fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, cuttHipMbar& mb) {
   std::memset(&mb, 0, sizeof(mb));
   int n = 0;
-  for (int r = 0; r < pb.rank; r++) {
+  for (int i = 0; i < pb.rank; i++) {
+    const int r = mbarOrder == 1 ? pb.perm[i] : i;
     if (inMmk[r]) continue;
     mb.d[n].extent = (uint32_t)pb.dim[r];
     mb.d[n].strideIn = (uint32_t)pb.strideIn[r];
@@ -253,44 +259,56 @@ void fillMbar(const Problem& pb, const std::vector<char>& inMmk, cuttHipMbar& mb
   mb.n = n;
 }
 
-// Extent of rank r inside one staged block of slab size `slab`.
-inline int blockExtent(const Split& sp, const Problem& pb, int r, int slab) {
-  return r == sp.splitRank ? slab : pb.dim[r];
+// Extent of rank r inside one staged block whose split ranks have the slab sizes slab[0..1].
+inline int blockExtent(const Split& sp, const Problem& pb, int r, const int* slab) {
+  const int slot = sp.splitSlot(r);
+  return slot >= 0 ? slab[slot] : pb.dim[r];
 }
 
 // Geometry of one slab class: volume and contiguous run lengths.
-void classGeometry(const Split& sp, const Problem& pb, int slab, int& vol, int& inCont, int& outCont) {
+void classGeometry(const Split& sp, const Problem& pb, const int* slab, int64_t& vol, int64_t& inCont,
+                   int64_t& outCont) {
   int64_t v = 1, ic = 1, oc = 1;
   for (int r = 0; r < pb.rank; r++)
     if (sp.inMmk[r]) v *= blockExtent(sp, pb, r, slab);
   for (int r = 0; r < pb.rank && sp.inMmk[r]; r++) {
     ic *= blockExtent(sp, pb, r, slab);
-    if (r == sp.splitRank) break;
+    if (sp.splitSlot(r) >= 0) break;
   }
   for (int j = 0; j < pb.rank && sp.inMmk[pb.perm[j]]; j++) {
     const int r = pb.perm[j];
     oc *= blockExtent(sp, pb, r, slab);
-    if (r == sp.splitRank) break;
+    if (sp.splitSlot(r) >= 0) break;
   }
-  vol = (int)v;
-  inCont = (int)ic;
-  outCont = (int)oc;
+  vol = v;
+  inCont = ic;
+  outCont = oc;
 }
 
-// Threads per workgroup for a staged block of `vol` elements that needs `lds` bytes.
-int choosePackedThreads(int64_t vol, size_t lds, const cuttHipDeviceProps& props) {
-  const int64_t byLds = std::max<int64_t>(1, (int64_t)(props.ldsPerCU / std::max<size_t>(lds, 1)));
-  // Fill the CU's thread slots with the workgroups that fit by LDS ...
-  int64_t nt = (props.maxThreadsPerCU / std::min<int64_t>(byLds, 8)) / 64 * 64;
-  // ... but keep at least ~4 elements per lane, and stay inside the hardware limit.
-  nt = std::min<int64_t>(nt, roundUp64(ceilDiv(vol, 4)));
-  nt = std::min<int64_t>(nt, props.maxThreadsPerBlock);
-  nt = std::max<int64_t>(nt, 64);
-  return (int)nt;
+// Which of the four slab-size classes a plan uses: bit i of c set = split rank i has its larger slab.
+inline bool classUsed(const cuttHipPackedArgs& a, int c) {
+  return !((c & 1) && a.split[0].slabRem == 0) && !((c & 2) && a.split[1].slabRem == 0);
+}
+
+// Threads per workgroup and elements per lane (1, 2, 4, 8) for a staged block of `vol`
+// elements.  numThreads = 0: does not fit.  Eight elements per lane is the most the kernel keeps
+// in registers without losing occupancy (three table words and one data word per element).
+constexpr int kMaxElemsPerThread = 8;
+
+void choosePackedThreads(int64_t vol, const cuttHipDeviceProps& props, int& numThreads,
+                         int& elemsPerThread) {
+  numThreads = 0;
+  elemsPerThread = 0;
+  int e = vol > 4096 ? 8 : (vol > 512 ? 4 : (vol > 128 ? 2 : 1));
+  while (e < kMaxElemsPerThread && roundUp64(ceilDiv(vol, e)) > props.maxThreadsPerBlock) e *= 2;
+  const int64_t nt = roundUp64(ceilDiv(vol, e));
+  if (nt > props.maxThreadsPerBlock) return;
+  numThreads = (int)nt;
+  elemsPerThread = e;
 }
 
 // Fill the launch geometry of a Packed / PackedSplit candidate.  False = does not fit.
-bool setupPacked(Plan& plan, const cuttHipDeviceProps& props) {
+bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptions& opt) {
   const Split& sp = plan.split;
   const Problem& pb = plan.pb;
   cuttHipPackedArgs& a = plan.packed;
@@ -298,52 +316,85 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props) {
   a.elemSize = pb.elemSize;
   a.volMbar = (int)sp.volMbar;
   a.padShift = kPadShift;
-  if (sp.method == kPackedSplit) {
-    a.numSplit = sp.numSplit;
-    a.slabFloor = sp.splitDim / sp.numSplit;
-    a.slabRem = sp.splitDim % sp.numSplit;
-    a.splitStrideIn = (uint32_t)pb.strideIn[sp.splitRank];
-    a.splitStrideOut = (uint32_t)pb.strideOut[sp.splitRank];
-    if (a.slabFloor < 1) return false;
-  } else {
-    a.numSplit = 1;
-    a.slabFloor = 0;
-    a.slabRem = 0;
+  for (int i = 0; i < 2; i++) {
+    cuttHipSplitRank& sr = a.split[i];
+    sr.numSplit = 1;
+    if (sp.method == kPackedSplit && sp.splitRank[i] >= 0) {
+      sr.numSplit = sp.numSplit[i];
+      sr.slabFloor = sp.splitDim[i] / sp.numSplit[i];
+      sr.slabRem = sp.splitDim[i] % sp.numSplit[i];
+      sr.strideIn = (uint32_t)pb.strideIn[sp.splitRank[i]];
+      sr.strideOut = (uint32_t)pb.strideOut[sp.splitRank[i]];
+      if (sr.slabFloor < 1) return false;
+    }
   }
-  const int ncls = a.slabRem > 0 ? 2 : 1;
-  for (int c = 0; c < ncls; c++) {
-    int vol, ic, oc;
-    classGeometry(sp, pb, a.slabFloor + c, vol, ic, oc);
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(a, c)) continue;
+    const int slab[2] = {a.split[0].slabFloor + (c & 1), a.split[1].slabFloor + ((c >> 1) & 1)};
+    int64_t vol, ic, oc;
+    classGeometry(sp, pb, slab, vol, ic, oc);
+    if (vol > kMaxLdsSlots) return false;
     cuttHipPackedClass& k = a.cls[c];
-    k.vol = vol;
-    k.inCont = ic;
-    k.outCont = oc;
-    k.inMagic = divMagic((uint32_t)ic);
-    k.outMagic = divMagic((uint32_t)oc);
-    k.nRowsIn = vol / ic;
-    k.nRowsOut = vol / oc;
-    a.maxVol = std::max(a.maxVol, vol);
-    a.maxRowsIn = std::max(a.maxRowsIn, k.nRowsIn);
-    a.maxRowsOut = std::max(a.maxRowsOut, k.nRowsOut);
+    k.vol = (int)vol;
+    k.inCont = (int)ic;
+    k.outCont = (int)oc;
+    a.maxVol = std::max(a.maxVol, k.vol);
   }
   const int64_t slots = paddedSlots(a.maxVol);
   if (slots > kMaxLdsSlots) return false;
   a.ldsElems = (int)slots;
   plan.ldsBytes = cuttHipPackedLdsBytes(&a);
   if (plan.ldsBytes > props.ldsPerBlock) return false;
-  a.numThreads = choosePackedThreads(a.maxVol, plan.ldsBytes, props);
+  choosePackedThreads(a.maxVol, props, a.numThreads, a.elemsPerThread);
+  if (a.numThreads == 0) return false;
   // Work items per workgroup: amortise the table load without starving the chip of workgroups.
-  const int64_t items = sp.volMbar * (int64_t)a.numSplit;
+  const int64_t items = sp.volMbar * (int64_t)a.split[0].numSplit * a.split[1].numSplit;
   if (items > 0x7fffffffll) return false;
   const int64_t residentPerCU =
       std::max<int64_t>(1, std::min<int64_t>((int64_t)(props.ldsPerCU / plan.ldsBytes),
                                              props.maxThreadsPerCU / a.numThreads));
-  const int64_t wanted = (int64_t)props.cuCount * residentPerCU * 8;
-  a.itemsPerBlock = (int)std::max<int64_t>(1, std::min<int64_t>(8, items / std::max<int64_t>(wanted, 1)));
+  // Enough workgroups for several waves of residents, but several items each where possible: the
+  // table slice a workgroup loads is reused by all of its items.
+  const int64_t wanted = (int64_t)props.cuCount * residentPerCU * 4;
+  a.itemsPerBlock = (int)std::max<int64_t>(1, std::min<int64_t>(opt.maxItemsPerBlock, items / std::max<int64_t>(wanted, 1)));
   plan.numBlocks = ceilDiv(items, a.itemsPerBlock);
+  if (opt.xcdAware && plan.numBlocks >= 64) {
+    a.xcdChunk = (uint32_t)ceilDiv(plan.numBlocks, kNumXcd);
+    plan.numBlocks = (int64_t)a.xcdChunk * kNumXcd;
+  }
   plan.numThreads = a.numThreads;
-  fillMbar(pb, sp.inMmk, a.mbar);
+  fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
   return true;
+}
+
+// Ordering of a tiled launch: fills order, super-tile shape and the per-XCD chunk; returns the
+// number of workgroups.
+struct TileOrdering {
+  int order;
+  uint32_t xcdChunk, superM, superK;
+};
+
+int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
+                    TileOrdering& o) {
+  o.order = opt.tiledOrder >= 0 ? opt.tiledOrder : 3;
+  // Super-tiles of up to superM x superK tiles, shrunk where a direction has fewer tiles.
+  int64_t sm = std::min<int64_t>(opt.superM, tilesM), sk = std::min<int64_t>(opt.superK, tilesK);
+  // Equal-sized super-tiles: no nearly empty last one (its padding workgroups would leave XCDs idle).
+  sm = ceilDiv(tilesM, ceilDiv(tilesM, sm));
+  sk = ceilDiv(tilesK, ceilDiv(tilesK, sk));
+  o.superM = (uint32_t)sm;
+  o.superK = (uint32_t)sk;
+  int64_t logical = tilesM * tilesK * volMbar;
+  if (o.order >= 3) logical = ceilDiv(tilesM, sm) * ceilDiv(tilesK, sk) * sm * sk * volMbar;
+  o.xcdChunk = 0;
+  if (opt.xcdAware && logical >= 64) {
+    int64_t chunk = ceilDiv(logical, kNumXcd);
+    if (chunk * kNumXcd <= 0x7fffffffll) {
+      o.xcdChunk = (uint32_t)chunk;
+      return chunk * kNumXcd;
+    }
+  }
+  return logical;
 }
 
 bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptions& opt) {
@@ -363,9 +414,10 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.tilesM = (int)tilesM;
     a.tilesK = (int)ceilDiv(sp.volMk, kTile);
     a.volMbar = (int)sp.volMbar;
-    a.order = opt.tiledOrder >= 0 ? opt.tiledOrder : 0;
-    fillMbar(pb, sp.inMmk, a.mbar);
-    plan.numBlocks = (int64_t)a.tilesM * a.tilesK * sp.volMbar;
+    TileOrdering o;
+    plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
+    a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
+    fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
     plan.ldsBytes = (size_t)kTile * (kTile + 1) * pb.elemSize;
   } else {
     cuttHipTiledCopyArgs& a = plan.tcopy;
@@ -379,9 +431,10 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.tilesM = (int)tilesM;
     a.tilesK = (int)ceilDiv(sp.volMkBar, kTile);
     a.volMbar = (int)sp.volMbar;
-    a.order = opt.tiledOrder >= 0 ? opt.tiledOrder : 1;
-    fillMbar(pb, sp.inMmk, a.mbar);
-    plan.numBlocks = (int64_t)a.tilesM * a.tilesK * sp.volMbar;
+    TileOrdering o;
+    plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
+    a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
+    fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
     plan.ldsBytes = 0;
   }
   plan.numThreads = 256;
@@ -453,42 +506,61 @@ void addPacked(const Problem& pb, bool fromReduced, const cuttHipDeviceProps& pr
       p.method = p.split.method = kPacked;
       p.split.update(numMm, numMk, pb);
       if (p.split.volMmk > kMaxLdsSlots) break;  // larger numMk only grows the block
-      if (!setupPacked(p, props)) break;
+      if (!setupPacked(p, props, opt)) break;
       if (!exists(p.split, plans)) plans.push_back(std::move(p));
     }
   }
 }
 
-// Slab counts worth trying for a block that is too large for one workgroup.
-std::vector<int> splitCounts(const Split& sp, const Problem& pb, const cuttHipDeviceProps& props) {
-  std::vector<int> out;
-  const int64_t unsplitBytes = sp.volMmkUnsplit * pb.elemSize;
-  const int splitDim = sp.splitDim;
-  // Target staged sizes (data bytes): a quarter, a half and the whole of what one workgroup may hold
-  // beside its tables.
-  const int64_t cap = (int64_t)props.ldsPerBlock * pb.elemSize / (pb.elemSize + 3);
-  const int64_t targets[3] = {cap / 8, cap / 4, cap / 2};
-  for (int64_t t : targets) {
-    int64_t slab = t / std::max<int64_t>(unsplitBytes, 1);
-    if (slab < 2) slab = 2;
-    if (slab > splitDim / 2) slab = splitDim / 2;
-    if (slab < 2) continue;
-    // Prefer slab sizes that cover whole 128-byte lines when the split rank is contiguous on
-    // either side, and slab counts that divide the rank evenly.
-    const int lineElems = 128 / pb.elemSize;
-    int64_t best = slab;
-    if (slab >= lineElems) best = slab / lineElems * lineElems;
-    int ns = (int)ceilDiv(splitDim, best);
-    // the slab the kernel uses is ceil(splitDim/ns); nudge ns so that it stays <= slab
-    while (ns < splitDim && ceilDiv(splitDim, ns) > slab) ns++;
-    if (ns >= 2 && std::find(out.begin(), out.end(), ns) == out.end()) out.push_back(ns);
-  }
-  return out;
+// Staged-block sizes (in elements) worth trying when Mmk has to be cut: about an eighth, a
+// quarter and a half of what one workgroup's LDS holds beside its tables.
+std::vector<int64_t> stagedTargets(const Problem& pb, const cuttHipDeviceProps& props) {
+  // what one workgroup can stage: LDS, and kMaxElemsPerThread elements on each of its lanes
+  const int64_t cap = std::min<int64_t>({(int64_t)props.ldsPerBlock * 31 / 32 / pb.elemSize,
+                                         (int64_t)kMaxElemsPerThread * props.maxThreadsPerBlock, kMaxLdsSlots * 31 / 32});
+  return {cap / 4, cap / 2, cap};
+}
+
+// Number of slabs that cuts a rank of extent `dim` into slabs of at most `slab` entries.  One
+// entry of the rank spans `unit` contiguous elements; where possible the slab is rounded down so
+// that unit*slab is a whole number of 128-byte lines.
+int slabCount(int dim, int64_t slab, int64_t unit, int elemSize) {
+  if (slab < 1) slab = 1;
+  if (slab >= dim) return 1;
+  const int64_t lineElems = 128 / elemSize;
+  // entries per slab so that unit*entries is a multiple of a line
+  int64_t step = lineElems;
+  for (int64_t g = unit % lineElems; g; ) { const int64_t t = step % g; step = g; g = t; }  // gcd(unit, lineElems)
+  step = lineElems / step;
+  if (slab >= step) slab = slab / step * step;
+  int ns = (int)ceilDiv(dim, slab);
+  while (ns < dim && ceilDiv(dim, ns) > slab) ns++;
+  return ns;
+}
+
+// Try one PackedSplit geometry; adds it when it fits and is new.  Returns true if it fits.
+bool tryPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProps& props,
+                    const PlannerOptions& opt, int numMm, int numMk, int rank0, int ns0, int rank1,
+                    int ns1, std::vector<Plan>& plans) {
+  Plan p;
+  p.pb = pb;
+  p.fromReduced = fromReduced;
+  p.method = p.split.method = kPackedSplit;
+  int slot = 0;
+  if (rank0 >= 0 && ns0 > 1) { p.split.splitRank[slot] = rank0; p.split.numSplit[slot] = ns0; slot++; }
+  if (rank1 >= 0 && ns1 > 1 && rank1 != rank0) { p.split.splitRank[slot] = rank1; p.split.numSplit[slot] = ns1; slot++; }
+  if (slot == 0) return false;
+  p.split.update(numMm, numMk, pb);
+  if (p.split.volStaged() > kMaxLdsSlots) return false;
+  if (!setupPacked(p, props, opt)) return false;
+  if (!exists(p.split, plans)) plans.push_back(std::move(p));
+  return true;
 }
 
 void addPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProps& props,
                     const PlannerOptions& opt, std::vector<Plan>& plans) {
   if (!allowed(opt, kPackedSplit)) return;
+  const std::vector<int64_t> targets = stagedTargets(pb, props);
   for (int numMm = 1; numMm < pb.rank; numMm++) {
     for (int numMk = 1; numMk < pb.rank; numMk++) {
       Split base;
@@ -500,34 +572,64 @@ void addPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProp
         probe.pb = pb;
         probe.method = probe.split.method = kPacked;
         probe.split = base;
-        if (base.volMmk <= kMaxLdsSlots && setupPacked(probe, props)) continue;
+        if (base.volMmk <= kMaxLdsSlots && setupPacked(probe, props, opt)) continue;
       }
-      // Split the largest rank of Mmk (first one wins ties, input ranks before output ranks).
-      int splitRank = -1, maxDim = 0;
-      for (int r = 0; r < numMm; r++)
-        if (pb.dim[r] > maxDim) { maxDim = pb.dim[r]; splitRank = r; }
-      for (int j = 0; j < numMk; j++)
-        if (pb.dim[pb.perm[j]] > maxDim) { maxDim = pb.dim[pb.perm[j]]; splitRank = pb.perm[j]; }
-      if (splitRank < 0 || maxDim < 4) break;
-      base.method = kPackedSplit;
-      base.splitRank = splitRank;
-      base.numSplit = 1;
-      base.update(numMm, numMk, pb);
-      // Even slabs of two entries must fit, otherwise larger numMk cannot fit either.
-      if (paddedSlots(2 * base.volMmkUnsplit) > kMaxLdsSlots) break;
       bool any = false;
-      for (int ns : splitCounts(base, pb, props)) {
-        Plan p;
-        p.pb = pb;
-        p.fromReduced = fromReduced;
-        p.method = kPackedSplit;
-        p.split = base;
-        p.split.numSplit = ns;
-        p.split.update(numMm, numMk, pb);
-        if (!setupPacked(p, props)) continue;
-        any = true;
-        if (!exists(p.split, plans)) plans.push_back(std::move(p));
+      // (a) Cut the largest rank of Mmk (the reference's choice, src/cuttplan.cpp:580-596).
+      {
+        int big = -1, maxDim = 0;
+        for (int r = 0; r < numMm; r++)
+          if (pb.dim[r] > maxDim) { maxDim = pb.dim[r]; big = r; }
+        for (int j = 0; j < numMk; j++)
+          if (pb.dim[pb.perm[j]] > maxDim) { maxDim = pb.dim[pb.perm[j]]; big = pb.perm[j]; }
+        if (big >= 0 && maxDim >= 4) {
+          const int64_t unsplit = base.volMmk / maxDim;
+          // contiguous elements per entry of the rank, if it continues a contiguous run
+          for (int64_t t : targets) {
+            int64_t slab = std::max<int64_t>(2, t / std::max<int64_t>(unsplit, 1));
+            slab = std::min<int64_t>(slab, maxDim / 2);
+            if (slab < 2) continue;
+            const int ns = slabCount(maxDim, slab, unsplit, pb.elemSize);
+            if (ns >= 2 && tryPackedSplit(pb, fromReduced, props, opt, numMm, numMk, big, ns, -1, 1, plans))
+              any = true;
+          }
+        }
       }
+      // (b) Cut the last rank of the input-contiguous set and the last rank of the
+      // output-contiguous set: a 2-D tile over the fused rank sets, with balanced run lengths.
+      {
+        const int rM = numMm - 1, rK = pb.perm[numMk - 1];
+        const int dM = pb.dim[rM], dK = pb.dim[rK];
+        int64_t baseIn = 1, baseOut = 1;
+        for (int r = 0; r < rM; r++) baseIn *= pb.dim[r];
+        for (int j = 0; j < numMk - 1; j++) baseOut *= pb.dim[pb.perm[j]];
+        if (rM == rK) {
+          // one rank ends both runs: covered by (a) when it is the largest; else cut it alone
+          const int64_t unsplit = base.volMmk / dM;
+          for (int64_t t : targets) {
+            const int64_t slab = std::min<int64_t>(std::max<int64_t>(1, t / std::max<int64_t>(unsplit, 1)), dM);
+            const int ns = slabCount(dM, slab, baseIn, pb.elemSize);
+            if (ns >= 2 && tryPackedSplit(pb, fromReduced, props, opt, numMm, numMk, rM, ns, -1, 1, plans))
+              any = true;
+          }
+        } else {
+          const int64_t other = base.volMmk / ((int64_t)dM * dK);
+          for (int64_t t : targets) {
+            const double avail = (double)t / (double)other;  // budget for slabM * slabK
+            if (avail < 1.0) continue;
+            // balance the run lengths baseIn*slabM and baseOut*slabK
+            double sM = std::sqrt(avail * (double)baseOut / (double)baseIn);
+            sM = std::min<double>(std::max(1.0, sM), dM);
+            double sK = std::min<double>(std::max(1.0, avail / sM), dK);
+            sM = std::min<double>(std::max(1.0, avail / sK), dM);
+            const int nsM = slabCount(dM, (int64_t)sM, baseIn, pb.elemSize);
+            const int nsK = slabCount(dK, (int64_t)sK, baseOut, pb.elemSize);
+            if (nsM == 1 && nsK == 1) continue;
+            if (tryPackedSplit(pb, fromReduced, props, opt, numMm, numMk, rM, nsM, rK, nsK, plans)) any = true;
+          }
+        }
+      }
+      // Neither cut fits: a larger numMk only grows the block.
       if (!any) break;
     }
   }
@@ -558,14 +660,15 @@ bool Plan::buildTables() {
     return true;
   }
   const Split& sp = split;
-  const int ncls = packed.slabRem > 0 ? 2 : 1;
-  for (int c = 0; c < ncls; c++) {
-    const int slab = packed.slabFloor + c;
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(packed, c)) continue;
+    const int slab[2] = {packed.split[0].slabFloor + (c & 1), packed.split[1].slabFloor + ((c >> 1) & 1)};
     PackedTables& t = tab[c];
     t.vol = packed.cls[c].vol;
     t.inCont = packed.cls[c].inCont;
     t.outCont = packed.cls[c].outCont;
-    // Ranks of Mmk in input order with their in-compact strides.
+    // Ranks of Mmk in input order with their in-compact strides.  The leading ranks up to and
+    // including the first split rank form the contiguous row; the others enumerate the rows.
     std::vector<int64_t> compactIn(pb.rank, 0);
     int64_t cstride = 1;
     std::vector<RadixDim> rowsIn;
@@ -579,7 +682,7 @@ bool Plan::buildTables() {
       compactIn[r] = cstride;
       cstride *= e;
       if (!inPrefix) rowsIn.push_back({e, pb.strideIn[r]});
-      if (r == sp.splitRank) inPrefix = false;  // ranks after the split rank start new rows
+      if (sp.splitSlot(r) >= 0) inPrefix = false;  // ranks after a split rank start new rows
     }
     if (cstride != t.vol) return false;
     enumerateOffsets(rowsIn, t.vol / t.inCont, t.rowIn);
@@ -595,13 +698,20 @@ bool Plan::buildTables() {
       const int e = blockExtent(sp, pb, r, slab);
       gather.push_back({e, compactIn[r]});
       if (!outPrefix) rowsOut.push_back({e, pb.strideOut[r]});
-      if (r == sp.splitRank) outPrefix = false;
+      if (sp.splitSlot(r) >= 0) outPrefix = false;
     }
     enumerateOffsets(rowsOut, t.vol / t.outCont, t.rowOut);
     std::vector<uint32_t> pos;
     enumerateOffsets(gather, t.vol, pos);
     t.shIdx.resize(pos.size());
     for (size_t q = 0; q < pos.size(); q++) t.shIdx[q] = (uint16_t)(pos[q] + (pos[q] >> packed.padShift));
+    // Per-element offsets: row offset + column inside the contiguous run.
+    t.inOff.resize((size_t)t.vol);
+    t.outOff.resize((size_t)t.vol);
+    for (int p = 0; p < t.vol; p++) {
+      t.inOff[(size_t)p] = t.rowIn[(size_t)(p / t.inCont)] + (uint32_t)(p % t.inCont);
+      t.outOff[(size_t)p] = t.rowOut[(size_t)(p / t.outCont)] + (uint32_t)(p % t.outCont);
+    }
   }
   tablesBuilt = true;
   return true;
@@ -611,20 +721,21 @@ int Plan::activate() {
   if (method != kPacked && method != kPackedSplit) return 0;
   if (dTables) return 0;
   if (!buildTables()) return -1;
-  const int ncls = packed.slabRem > 0 ? 2 : 1;
-  // One allocation: [rowIn | rowOut | shIdx] per class, each piece 16-byte aligned.
+  // One allocation: [inOff | outOff | shIdx] per class, each piece 16-byte aligned.
   auto align16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
   size_t total = 0;
-  size_t off[2][3];
-  for (int c = 0; c < ncls; c++) {
-    off[c][0] = total; total += align16(tab[c].rowIn.size() * sizeof(uint32_t));
-    off[c][1] = total; total += align16(tab[c].rowOut.size() * sizeof(uint32_t));
+  size_t off[4][3] = {};
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(packed, c)) continue;
+    off[c][0] = total; total += align16(tab[c].inOff.size() * sizeof(uint32_t));
+    off[c][1] = total; total += align16(tab[c].outOff.size() * sizeof(uint32_t));
     off[c][2] = total; total += align16(tab[c].shIdx.size() * sizeof(uint16_t));
   }
   std::vector<unsigned char> host(total, 0);
-  for (int c = 0; c < ncls; c++) {
-    std::memcpy(&host[off[c][0]], tab[c].rowIn.data(), tab[c].rowIn.size() * sizeof(uint32_t));
-    std::memcpy(&host[off[c][1]], tab[c].rowOut.data(), tab[c].rowOut.size() * sizeof(uint32_t));
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(packed, c)) continue;
+    std::memcpy(&host[off[c][0]], tab[c].inOff.data(), tab[c].inOff.size() * sizeof(uint32_t));
+    std::memcpy(&host[off[c][1]], tab[c].outOff.data(), tab[c].outOff.size() * sizeof(uint32_t));
     std::memcpy(&host[off[c][2]], tab[c].shIdx.data(), tab[c].shIdx.size() * sizeof(uint16_t));
   }
   void* d = nullptr;
@@ -636,10 +747,11 @@ int Plan::activate() {
     return e;
   }
   dTables = d;
-  for (int c = 0; c < ncls; c++) {
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(packed, c)) continue;
     unsigned char* base = (unsigned char*)d;
-    packed.cls[c].rowIn = (const uint32_t*)(base + off[c][0]);
-    packed.cls[c].rowOut = (const uint32_t*)(base + off[c][1]);
+    packed.cls[c].inOff = (const uint32_t*)(base + off[c][0]);
+    packed.cls[c].outOff = (const uint32_t*)(base + off[c][1]);
     packed.cls[c].shIdx = (const uint16_t*)(base + off[c][2]);
   }
   return 0;
@@ -668,7 +780,8 @@ std::string Plan::describe() const {
     << " numMk " << split.numMk << " volMmk " << split.volMmk << " volMbar " << split.volMbar
     << " inCont " << split.volMmkInCont << " outCont " << split.volMmkOutCont;
   if (method == kPackedSplit)
-    s << " splitRank " << split.splitRank << " numSplit " << split.numSplit;
+    s << " splitRank " << split.splitRank[0] << "/" << split.splitRank[1] << " numSplit " << split.numSplit[0]
+      << "/" << split.numSplit[1];
   s << " blocks " << numBlocks << " threads " << numThreads << " lds " << ldsBytes;
   if (method == kPacked || method == kPackedSplit) s << " items/block " << packed.itemsPerBlock;
   s << " predicted_us " << model.usPredicted;

@@ -53,22 +53,27 @@ struct Split {
   int sizeMmk = 0, sizeMbar = 0, sizeMkBar = 0;
   int64_t volMm = 0, volMk = 0, volMmk = 0, volMkBar = 0, volMbar = 0;
   int64_t volMmkInCont = 0, volMmkOutCont = 0;  // for the largest slab when split
-  // PackedSplit
-  int splitRank = -1;
-  int splitDim = 0;
-  int numSplit = 1;
+  // PackedSplit: up to two ranks of Mmk are cut into slabs (slot 0 first; an unused slot has
+  // splitRank -1 and numSplit 1)
+  int splitRank[2] = {-1, -1};
+  int splitDim[2] = {0, 0};
+  int numSplit[2] = {1, 1};
   int64_t volMmkUnsplit = 0;
   std::vector<char> inMmk;  // per input rank
 
   void update(int numMm, int numMk, const Problem& pb);
-  int slabMax() const { return splitRank < 0 ? 0 : (splitDim + numSplit - 1) / numSplit; }
+  int slabMax(int i) const { return splitRank[i] < 0 ? 1 : (splitDim[i] + numSplit[i] - 1) / numSplit[i]; }
+  int splitSlot(int rank) const { return rank == splitRank[0] ? 0 : (rank == splitRank[1] ? 1 : -1); }
   int64_t volStaged() const;  // elements one workgroup stages at most
 };
 
-// Host copy of the index tables of one slab size (see cuttHipPackedClass).
+// Host copy of the index tables of one slab-size class.  rowIn/rowOut hold one offset per
+// contiguous run (the cost model walks those); inOff/outOff/shIdx are the per-element tables the
+// kernel reads (see cuttHipPackedClass).
 struct PackedTables {
   int vol = 0, inCont = 0, outCont = 0;
   std::vector<uint32_t> rowIn, rowOut;
+  std::vector<uint32_t> inOff, outOff;
   std::vector<uint16_t> shIdx;
 };
 
@@ -99,7 +104,7 @@ struct Plan {
   int numThreads = 0;
 
   // Packed host tables, built on demand (buildTables) and device copies (activate).
-  PackedTables tab[2];
+  PackedTables tab[4];
   bool tablesBuilt = false;
   void* dTables = nullptr;
 
@@ -121,7 +126,11 @@ struct Plan {
 
 struct PlannerOptions {
   int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
-  int tiledOrder = -1;      // -1 = planner's choice
+  int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
+  int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3/4: strips of 8 tiles along Mm
+  int maxItemsPerBlock = 16; // Packed/PackedSplit: work items one workgroup handles at most
+  int mbarOrder = 1;        // order of the Mbar ranks: 0 = input order, 1 = output order
+  bool xcdAware = true;     // give every XCD (private L2) a contiguous chunk of the workgroup sequence
 };
 
 // Build every candidate for the original and the fused problem

@@ -32,7 +32,8 @@ typedef struct cuttPlanInfo {
   int fromReduced;      /* 1 if built from the rank-fused problem */
   int rank;             /* rank of the problem the plan was built from */
   int numMm, numMk;
-  int splitRank, splitDim, numSplit;
+  int splitRank, splitDim, numSplit;     /* first split rank (PackedSplit), -1/0/1 if none */
+  int splitRank2, splitDim2, numSplit2;  /* second split rank, -1/0/1 if none */
   long long volMm, volMk, volMmk, volMbar, volMmkInCont, volMmkOutCont, volMmkUnsplit;
   long long numBlocks;
   int numThreads;
@@ -107,16 +108,18 @@ int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
 
 /*
  * Raw index data of candidate `index`, for checking a plan's address stream
- * on the host.  `what` selects the array, `cls` the slab class (0/1) where it
+ * on the host.  `what` selects the array, `cls` the slab class (0..3) where it
  * applies; the function copies up to maxCount 64-bit values into `values` and
  * returns the array's length (or -1).
  *
  *   what 0: Mbar table, 3 values per rank: extent, strideIn, strideOut
- *   what 1: tile geometry: volMm, volMk, strideInK, strideOut(M or K), tilesM, tilesK, volMbar, order
- *   what 2: packed scalars: numThreads, volMbar, numSplit, slabFloor, slabRem, splitStrideIn,
- *           splitStrideOut, itemsPerBlock, padShift, ldsElems
- *   what 3: class scalars: vol, inCont, outCont, inMagic, outMagic, nRowsIn, nRowsOut
- *   what 4: rowIn[]   what 5: rowOut[]   what 6: shIdx[]
+ *   what 1: tile geometry: volMm, volMk, strideInK, strideOut(M or K), tilesM, tilesK, volMbar, order,
+ *           xcdChunk, superM, superK
+ *   what 2: packed scalars: numThreads, volMbar, itemsPerBlock, padShift, ldsElems, xcdChunk,
+ *           elemsPerThread, then for each of the two split slots: numSplit, slabFloor, slabRem,
+ *           strideIn, strideOut
+ *   what 3: class scalars: vol, inCont, outCont
+ *   what 4: inOff[]   what 5: outOff[]   what 6: shIdx[]
  */
 long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                              long long maxCount);

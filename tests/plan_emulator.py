@@ -25,6 +25,44 @@ def _mbar_offsets(tab, vol_mbar):
     return off_in, off_out
 
 
+def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k):
+    """The kernels' workgroup-index decoding visits every (tile, Mbar position) exactly once."""
+    b = np.arange(num_blocks, dtype=np.int64)
+    if xcd_chunk:
+        assert num_blocks == 8 * xcd_chunk
+        l = (b % 8) * xcd_chunk + b // 8
+    else:
+        l = b
+    if order == 0:
+        t, m = l // vol_mbar, l % vol_mbar
+        tk, tm = t // tiles_m, t % tiles_m
+        ok = tk < tiles_k
+    elif order == 1:
+        t, tm = l // tiles_m, l % tiles_m
+        m, tk = t // tiles_k, t % tiles_k
+        ok = m < vol_mbar
+    elif order == 2:
+        t, tk = l // tiles_k, l % tiles_k
+        m, tm = t // tiles_m, t % tiles_m
+        ok = m < vol_mbar
+    else:
+        assert order in (3, 4) and sup_m >= 1 and sup_k >= 1
+        n_sm, n_sk = -(-tiles_m // sup_m), -(-tiles_k // sup_k)
+        per = sup_m * sup_k
+        w, t = l % per, l // per
+        st, m = t % (n_sm * n_sk), t // (n_sm * n_sk)
+        if order == 3:
+            tm = (st % n_sm) * sup_m + w % sup_m
+            tk = (st // n_sm) * sup_k + w // sup_m
+        else:
+            tk = (st % n_sk) * sup_k + w % sup_k
+            tm = (st // n_sk) * sup_m + w // sup_k
+        ok = (m < vol_mbar) & (tm < tiles_m) & (tk < tiles_k)
+    key = (m[ok] * tiles_k + tk[ok]) * tiles_m + tm[ok]
+    assert key.size == tiles_m * tiles_k * vol_mbar, "tile decode misses or repeats tiles"
+    assert np.array_equal(np.sort(key), np.arange(key.size))
+
+
 def emulate(cands, idx, data):
     """Return (out, write_count) for candidate idx applied to the flat array data."""
     info = cands.info(idx)
@@ -46,9 +84,9 @@ def emulate(cands, idx, data):
 
     mbar = cands.data(idx, 0)
     if name in ("Tiled", "TiledCopy"):
-        vol_mm, vol_mk, s_in_k, s_out, tiles_m, tiles_k, vol_mbar, order = [int(v) for v in cands.data(idx, 1)]
+        vol_mm, vol_mk, s_in_k, s_out, tiles_m, tiles_k, vol_mbar, order, xcd_chunk, sup_m, sup_k = [int(v) for v in cands.data(idx, 1)]
         assert tiles_m == -(-vol_mm // 64) and tiles_k == -(-vol_mk // 64)
-        assert info.numBlocks == tiles_m * tiles_k * vol_mbar
+        _check_tile_decode(info.numBlocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k)
         off_in, off_out = _mbar_offsets(mbar, vol_mbar)
         x = np.arange(vol_mm, dtype=np.int64)
         k = np.arange(vol_mk, dtype=np.int64)
@@ -63,30 +101,32 @@ def emulate(cands, idx, data):
         return out, count
 
     # Packed / PackedSplit
-    (num_threads, vol_mbar, num_split, slab_floor, slab_rem, split_in, split_out, items_per_block,
-     pad_shift, lds_elems) = [int(v) for v in cands.data(idx, 2)]
+    sc = [int(v) for v in cands.data(idx, 2)]
+    num_threads, vol_mbar, items_per_block, pad_shift, lds_elems, xcd_chunk, elems_per_thread = sc[:7]
+    splits = [sc[7:12], sc[12:17]]  # numSplit, slabFloor, slabRem, strideIn, strideOut
     assert num_threads % 64 == 0 and 64 <= num_threads <= 1024
+    assert elems_per_thread in (1, 2, 4, 8)
     off_in, off_out = _mbar_offsets(mbar, vol_mbar)
-    total_items = vol_mbar * num_split
-    assert info.numBlocks == -(-total_items // items_per_block)
+    ns0, ns1 = splits[0][0], splits[1][0]
+    total_items = vol_mbar * ns0 * ns1
+    logical_blocks = -(-total_items // items_per_block)
+    if xcd_chunk:
+        # workgroup b handles logical block (b % 8) * xcd_chunk + b // 8: every logical block once
+        assert info.numBlocks == 8 * xcd_chunk and 8 * xcd_chunk >= logical_blocks
+        b = np.arange(info.numBlocks, dtype=np.int64)
+        lb = (b % 8) * xcd_chunk + b // 8
+        assert np.array_equal(np.sort(lb), b)
+    else:
+        assert info.numBlocks == logical_blocks
     classes = {}
-    for c in ([0, 1] if slab_rem > 0 else [0]):
-        cvol, in_cont, out_cont, in_magic, out_magic, n_rows_in, n_rows_out = [int(v) for v in cands.data(idx, 3, c)]
-        row_in, row_out, sh = cands.data(idx, 4, c), cands.data(idx, 5, c), cands.data(idx, 6, c)
-        assert len(row_in) == n_rows_in and len(row_out) == n_rows_out and len(sh) == cvol
-        assert n_rows_in * in_cont == cvol and n_rows_out * out_cont == cvol
-        assert cvol <= 65536
-        p = np.arange(cvol, dtype=np.uint64)
-        # the kernel's division: mulhi(p, magic), or p itself when the divisor is 1
-        row_p = (p * np.uint64(in_magic)) >> np.uint64(32) if in_cont > 1 else p
-        row_q = (p * np.uint64(out_magic)) >> np.uint64(32) if out_cont > 1 else p
-        assert np.array_equal(row_p, p // np.uint64(in_cont)), "input magic division is wrong"
-        assert np.array_equal(row_q, p // np.uint64(out_cont)), "output magic division is wrong"
-        p = p.astype(np.int64)
-        row_p = row_p.astype(np.int64)
-        row_q = row_q.astype(np.int64)
-        in_off = row_in[row_p] + (p - row_p * in_cont)
-        out_off = row_out[row_q] + (p - row_q * out_cont)
+    for c in range(4):
+        if ((c & 1) and splits[0][2] == 0) or ((c & 2) and splits[1][2] == 0):
+            continue
+        cvol, in_cont, out_cont = [int(v) for v in cands.data(idx, 3, c)]
+        in_off, out_off, sh = cands.data(idx, 4, c), cands.data(idx, 5, c), cands.data(idx, 6, c)
+        assert len(in_off) == cvol and len(out_off) == cvol and len(sh) == cvol
+        assert cvol <= num_threads * elems_per_thread, "a lane would need more table registers"
+        p = np.arange(cvol, dtype=np.int64)
         slot = p + (p >> pad_shift)
         assert slot.max() < lds_elems, "LDS slot outside the buffer"
         assert len(np.unique(slot)) == cvol
@@ -98,9 +138,12 @@ def emulate(cands, idx, data):
         assert src_p.min() >= 0, "gather reads an LDS slot that was never written"
         classes[c] = (in_off[src_p], out_off)
     for w in range(total_items):
-        m, s = divmod(w, num_split)
-        c = 1 if s < slab_rem else 0
-        p0 = s * slab_floor + min(s, slab_rem)
+        t, s0 = divmod(w, ns0)
+        m, s1 = divmod(t, ns1)
+        c = (1 if s0 < splits[0][2] else 0) + (2 if s1 < splits[1][2] else 0)
+        p0 = s0 * splits[0][1] + min(s0, splits[0][2])
+        p1 = s1 * splits[1][1] + min(s1, splits[1][2])
         src_rel, dst_rel = classes[c]
-        scatter(off_out[m] + p0 * split_out + dst_rel, off_in[m] + p0 * split_in + src_rel)
+        scatter(off_out[m] + p0 * splits[0][4] + p1 * splits[1][4] + dst_rel,
+                off_in[m] + p0 * splits[0][3] + p1 * splits[1][3] + src_rel)
     return out, count
