@@ -140,6 +140,24 @@ int chooseHeuristic(const std::vector<Plan>& plans) {
   return best;
 }
 
+PlannerOptions plannerOptions(int forceMethod) {
+  PlannerOptions opt;
+  opt.forceMethod = forceMethod;
+  // Tuning knobs for experiments; the defaults are what the library ships with.
+  if (const char* e = std::getenv("CUTT_TILED_ORDER")) opt.tiledOrder = std::atoi(e);
+  if (const char* e = std::getenv("CUTT_XCD_AWARE")) opt.xcdAware = std::atoi(e) != 0;
+  if (const char* e = std::getenv("CUTT_ELEMS_PER_THREAD")) {
+    const int v = std::atoi(e);
+    if (v == 1 || v == 2 || v == 4 || v == 8) opt.elemsPerThread = v;
+  }
+  if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
+  if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));
+  return opt;
+}
+
 bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
                const cuttHipDeviceProps& props, int forceMethod, std::vector<Plan>& plans) {
   Problem orig, red;
@@ -147,16 +165,7 @@ bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
   std::vector<int> redDim, redPerm;
   reduceRanks(rank, dim, perm, redDim, redPerm);
   red.set((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType);
-  PlannerOptions opt;
-  opt.forceMethod = forceMethod;
-  // Tuning knobs for experiments; the defaults are what the library ships with.
-  if (const char* e = std::getenv("CUTT_TILED_ORDER")) opt.tiledOrder = std::atoi(e);
-  if (const char* e = std::getenv("CUTT_XCD_AWARE")) opt.xcdAware = std::atoi(e) != 0;
-  if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
-  if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
-  if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
-  if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));
-  return createPlans(orig, red, props, opt, plans);
+  return createPlans(orig, red, props, plannerOptions(forceMethod), plans);
 }
 
 cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int deviceID, int numCandidates,
@@ -227,12 +236,19 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   std::vector<Plan> plans;
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
   if (plans.empty()) return CUTT_INTERNAL_ERROR;
-  // The model's numbers are kept for reporting; they do not influence the choice.
   for (Plan& p : plans)
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
 
   size_t numBytes = sizeofType;
   for (int i = 0; i < rank; i++) numBytes *= (size_t)dim[i];
+
+  // Candidates the model puts far behind its best are not timed (its error is well inside that
+  // margin); CUTT_MEASURE_ALL=1 times every candidate, as the reference does.
+  double bestPred = 1e300;
+  for (const Plan& p : plans) bestPred = std::min(bestPred, p.model.usPredicted);
+  double margin = 1.6;
+  if (const char* e = std::getenv("CUTT_MEASURE_ALL"))
+    if (std::atoi(e) != 0) margin = 1e30;
 
   void *evStart = nullptr, *evStop = nullptr;
   if (cuttHipEventCreate(&evStart) != 0) return CUTT_INTERNAL_ERROR;
@@ -240,39 +256,79 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
     cuttHipEventDestroy(evStart);
     return CUTT_INTERNAL_ERROR;
   }
-  std::vector<double> us(plans.size(), 0.0);
-  int best = -1;
   double bestUs = 1e300;
   bool failed = false;
-  for (int i = 0; i < (int)plans.size() && !failed; i++) {
-    Plan& p = plans[i];
+  // Times plan p (two runs, the faster counts); returns false on a HIP error.
+  auto timePlan = [&](Plan& p, double& t) -> bool {
     p.stream = (void*)stream;
     p.deviceID = deviceID;
-    if (p.activate() != 0) { failed = true; break; }
-    double t = 1e300;
+    if (p.activate() != 0) return false;
+    t = 1e300;
     for (int rep = 0; rep < 2; rep++) {
       // Overwrite the output so that every run starts from the same cache state.
       if (cuttHipMemsetAsync(odata, 0xFF, numBytes, (void*)stream) != 0 ||
           cuttHipDeviceSynchronize() != 0 || cuttHipEventRecord(evStart, (void*)stream) != 0 ||
           p.launch(idata, odata) != 0 || cuttHipEventRecord(evStop, (void*)stream) != 0 ||
-          cuttHipEventSynchronize(evStop) != 0) {
-        failed = true;
-        break;
-      }
+          cuttHipEventSynchronize(evStop) != 0)
+        return false;
       float ms = 0;
-      if (cuttHipEventElapsedMs(evStart, evStop, &ms) != 0) { failed = true; break; }
+      if (cuttHipEventElapsedMs(evStart, evStop, &ms) != 0) return false;
       t = std::min(t, (double)ms * 1e3);
       if (t > 3.0 * bestUs) break;  // hopeless: do not spend a second run on it
     }
+    return true;
+  };
+
+  std::vector<double> us(plans.size(), 0.0);
+  int best = -1;
+  for (int i = 0; i < (int)plans.size() && !failed; i++) {
+    Plan& p = plans[i];
+    if (p.method != kTrivial && p.model.usPredicted > margin * bestPred) continue;
+    double t;
+    if (!timePlan(p, t)) { failed = true; break; }
     us[i] = t;
-    if (!failed && t < bestUs) {
+    if (t < bestUs) {
       bestUs = t;
+      if (best >= 0) plans[best].release();
       best = i;
+    } else {
+      p.release();
     }
-    if (i != best) p.release();
-    // a previous best that has been beaten no longer needs its tables
-    for (int j = 0; j < i; j++)
-      if (j != best) plans[j].release();
+  }
+  // Second stage: variants of the winner that differ only in workgroup ordering and granularity.
+  if (!failed && best >= 0 && plans[best].method != kTrivial) {
+    std::vector<PlannerOptions> variants;
+    const PlannerOptions base = plannerOptions(force);
+    if (plans[best].method == kTiled || plans[best].method == kTiledCopy) {
+      PlannerOptions v = base;
+      v.tiledOrder = 3; v.superM = 16; v.superK = 16;   // square patches instead of strips
+      variants.push_back(v);
+      v = base;
+      v.tiledOrder = 2;                                  // tiles along the output run fastest
+      variants.push_back(v);
+    } else {
+      for (int ipb : {1, 2, 8}) {
+        PlannerOptions v = base;
+        if (ipb == v.maxItemsPerBlock) continue;
+        v.maxItemsPerBlock = ipb;
+        variants.push_back(v);
+      }
+    }
+    for (const PlannerOptions& v : variants) {
+      Plan q;
+      if (!rebuildPlan(plans[best], props, v, q)) continue;
+      if (q.numBlocks == plans[best].numBlocks && q.method != kTiled && q.method != kTiledCopy) continue;
+      if (!estimatePlan(q, props, 10)) continue;
+      double t;
+      if (!timePlan(q, t)) { failed = true; break; }
+      if (t < bestUs) {
+        bestUs = t;
+        us.push_back(t);
+        plans[best].release();
+        plans.push_back(std::move(q));
+        best = (int)plans.size() - 1;
+      }
+    }
   }
   cuttHipEventDestroy(evStart);
   cuttHipEventDestroy(evStop);

@@ -291,26 +291,37 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   r.blocksPerCU = blocksPerCU;
 
   // --- time estimate ---
-  const double clockHz = props.clockKHz * 1e3;
-  const double cus = props.cuCount;
-  // Sustained HBM traffic: what a large device-to-device copy reaches on this part.
+  // The estimate is "time of a same-size device-to-device copy" times an overhead factor that is
+  // linear in a few transaction ratios.  The coefficients are a least-squares fit to the measured
+  // times of about 2600 candidates over 84 tensors of ~2e8 elements on one MI355X (ranks 2-7, 4- and
+  // 8-byte elements, timed by cuttPlanMeasure); on tensors left out of the fit the plan chosen by
+  // this estimate was on average 2 % and at worst 14 % slower than the measured best.
+  //  - Tiled / TiledCopy: workgroups on one XCD walk neighbouring tiles, so partly used lines are
+  //    found in the L2 and the line counts hardly matter; what costs is the padding of edge
+  //    tiles, whose clamped lanes repeat accesses that hit the L1 (about a quarter of a real one).
+  //  - Packed / PackedSplit: extra lines on the write side cost about twice as much as on the read
+  //    side (partly written lines have to be merged in the L2), 4-byte elements a little more per
+  //    byte than 8-byte ones, and a block cut into slabs a little more than a whole one.
   const double peakBW = (double)props.memClockKHz * 1e3 * 4.0 * (props.memBusWidthBits / 8.0);
-  const double sustainedBW = 0.64 * peakBW;
-  // Reads move whole lines; writes move the touched sectors, partial lines pay a merge penalty.
-  const double traffic = r.rdLines * kLineBytes + r.wrSectors * kSectorBytes +
-                         r.wrPartialLines * 64.0 + 0.25 * tableBytes;
-  const double tMem = traffic / sustainedBW;
-  // Address processing: a request costs at least 4 cycles, or one cycle per line it touches.
-  const double reqCycles = std::max(4.0 * (r.rdInstr + r.wrInstr), r.rdLines + r.wrLines);
-  const double tReq = reqCycles / (cus * clockHz);
-  const double tLds = r.ldsCycles / (cus * clockHz);
-  // Latency bound: bytes in flight per CU (4 loads per lane) against ~2 us loaded latency.
-  const double lanes = std::min((double)props.maxThreadsPerCU, blocksPerCU * plan.numThreads);
-  const double inflight = 0.5 * lanes * 4.0 * es * cus;  // half the waves are in their store phase
-  const double tLat = bytes / (inflight / 2.0e-6);
-  // Workgroup launch + barrier overhead.
-  const double tBlocks = (double)plan.numBlocks * 1.5e-6 / (cus * blocksPerCU);
-  const double t = std::max({tMem, tReq, tLat}) + 0.5 * tLds + tBlocks;
+  const double tCopy = 2.0 * bytes / (0.64 * peakBW);  // sustained rate of a large D2D copy
+  const double lineBytes = bytes / kLineBytes;
+  const double rdAmp = r.rdLines / lineBytes, wrAmp = r.wrLines / lineBytes;
+  const double partial = r.wrPartialLines / lineBytes;
+  double factor;
+  if (plan.method == kTiled || plan.method == kTiledCopy) {
+    const bool copy = plan.method == kTiledCopy;
+    const double tilesM = copy ? plan.tcopy.tilesM : plan.tiled.tilesM;
+    const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
+    const double waste = tilesM * tilesK * (double)plan.split.volMbar * kTile * kTile / (double)plan.pb.volume - 1.0;
+    factor = 1.03 + 0.30 * waste + (es == 4 ? 0.05 : 0.0) + (copy ? 0.15 : 0.0);
+  } else {
+    factor = 1.143 + 0.09 * (rdAmp - 1.0) + 0.22 * (wrAmp - 1.0) + 0.016 * partial + (es == 4 ? 0.04 : 0.0) -
+             (plan.method == kPacked ? 0.066 : 0.0);
+    // LDS bank conflicts of the gather, and table reloads when a block has few items.
+    factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
+    factor += 0.25 * tableBytes / (2.0 * bytes);
+  }
+  const double t = tCopy * factor;
   r.usPredicted = t * 1e6;
   return true;
 }

@@ -295,11 +295,13 @@ inline bool classUsed(const cuttHipPackedArgs& a, int c) {
 // in registers without losing occupancy (three table words and one data word per element).
 constexpr int kMaxElemsPerThread = 8;
 
-void choosePackedThreads(int64_t vol, const cuttHipDeviceProps& props, int& numThreads,
+void choosePackedThreads(int64_t vol, const cuttHipDeviceProps& props, int opt_e, int& numThreads,
                          int& elemsPerThread) {
   numThreads = 0;
   elemsPerThread = 0;
-  int e = vol > 4096 ? 8 : (vol > 512 ? 4 : (vol > 128 ? 2 : 1));
+  // As many elements per lane as the block allows: the loads a lane has in flight are what hides
+  // the memory latency, and smaller workgroups leave room for more of them on a CU.
+  int e = opt_e > 0 ? opt_e : (vol >= 512 ? 8 : (vol >= 256 ? 4 : (vol > 64 ? 2 : 1)));
   while (e < kMaxElemsPerThread && roundUp64(ceilDiv(vol, e)) > props.maxThreadsPerBlock) e *= 2;
   const int64_t nt = roundUp64(ceilDiv(vol, e));
   if (nt > props.maxThreadsPerBlock) return;
@@ -345,7 +347,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   a.ldsElems = (int)slots;
   plan.ldsBytes = cuttHipPackedLdsBytes(&a);
   if (plan.ldsBytes > props.ldsPerBlock) return false;
-  choosePackedThreads(a.maxVol, props, a.numThreads, a.elemsPerThread);
+  choosePackedThreads(a.maxVol, props, opt.elemsPerThread, a.numThreads, a.elemsPerThread);
   if (a.numThreads == 0) return false;
   // Work items per workgroup: amortise the table load without starving the chip of workgroups.
   const int64_t items = sp.volMbar * (int64_t)a.split[0].numSplit * a.split[1].numSplit;
@@ -355,8 +357,14 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
                                              props.maxThreadsPerCU / a.numThreads));
   // Enough workgroups for several waves of residents, but several items each where possible: the
   // table slice a workgroup loads is reused by all of its items.
-  const int64_t wanted = (int64_t)props.cuCount * residentPerCU * 4;
-  a.itemsPerBlock = (int)std::max<int64_t>(1, std::min<int64_t>(opt.maxItemsPerBlock, items / std::max<int64_t>(wanted, 1)));
+  if (opt.packedRounds > 0) {
+    // exactly `packedRounds` waves of resident workgroups, each with an equal share of the items
+    const int64_t target = (int64_t)props.cuCount * residentPerCU * opt.packedRounds;
+    a.itemsPerBlock = (int)std::max<int64_t>(1, ceilDiv(items, target));
+  } else {
+    const int64_t wanted = (int64_t)props.cuCount * residentPerCU * 4;
+    a.itemsPerBlock = (int)std::max<int64_t>(1, std::min<int64_t>(opt.maxItemsPerBlock, items / std::max<int64_t>(wanted, 1)));
+  }
   plan.numBlocks = ceilDiv(items, a.itemsPerBlock);
   if (opt.xcdAware && plan.numBlocks >= 64) {
     a.xcdChunk = (uint32_t)ceilDiv(plan.numBlocks, kNumXcd);
@@ -617,15 +625,22 @@ void addPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProp
           for (int64_t t : targets) {
             const double avail = (double)t / (double)other;  // budget for slabM * slabK
             if (avail < 1.0) continue;
-            // balance the run lengths baseIn*slabM and baseOut*slabK
-            double sM = std::sqrt(avail * (double)baseOut / (double)baseIn);
-            sM = std::min<double>(std::max(1.0, sM), dM);
-            double sK = std::min<double>(std::max(1.0, avail / sM), dK);
-            sM = std::min<double>(std::max(1.0, avail / sK), dM);
-            const int nsM = slabCount(dM, (int64_t)sM, baseIn, pb.elemSize);
-            const int nsK = slabCount(dK, (int64_t)sK, baseOut, pb.elemSize);
-            if (nsM == 1 && nsK == 1) continue;
-            if (tryPackedSplit(pb, fromReduced, props, opt, numMm, numMk, rM, nsM, rK, nsK, plans)) any = true;
+            // Slab of the input-side rank: (0) balance the run lengths baseIn*slabM and
+            // baseOut*slabK; (1), (2) keep the read runs at one or two 128-byte lines and give
+            // the rest of the budget to the write runs - partly written lines cost more than
+            // partly read ones, which the neighbouring workgroup finds in the L2.
+            const double lineElems = 128.0 / pb.elemSize;
+            const double choices[3] = {std::sqrt(avail * (double)baseOut / (double)baseIn),
+                                       lineElems / (double)baseIn, 2.0 * lineElems / (double)baseIn};
+            for (double sM : choices) {
+              sM = std::min<double>(std::max(1.0, std::ceil(sM)), dM);
+              const double sK = std::min<double>(std::max(1.0, avail / sM), dK);
+              sM = std::min<double>(std::max(1.0, avail / sK), dM);
+              const int nsM = slabCount(dM, (int64_t)sM, baseIn, pb.elemSize);
+              const int nsK = slabCount(dK, (int64_t)sK, baseOut, pb.elemSize);
+              if (nsM == 1 && nsK == 1) continue;
+              if (tryPackedSplit(pb, fromReduced, props, opt, numMm, numMk, rM, nsM, rK, nsK, plans)) any = true;
+            }
           }
         }
       }
@@ -636,6 +651,24 @@ void addPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProp
 }
 
 }  // namespace
+
+bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const PlannerOptions& opt, Plan& out) {
+  out = Plan();
+  out.method = src.method;
+  out.split = src.split;
+  out.pb = src.pb;
+  out.fromReduced = src.fromReduced;
+  switch (src.method) {
+    case kTiled:
+    case kTiledCopy:
+      return setupTiled(out, props, opt);
+    case kPacked:
+    case kPackedSplit:
+      return setupPacked(out, props, opt);
+    default:
+      return false;
+  }
+}
 
 bool createPlans(const Problem& orig, const Problem& red, const cuttHipDeviceProps& props,
                  const PlannerOptions& opt, std::vector<Plan>& plans) {

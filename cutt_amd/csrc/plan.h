@@ -128,7 +128,9 @@ struct PlannerOptions {
   int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
   int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3/4: strips of 8 tiles along Mm
-  int maxItemsPerBlock = 16; // Packed/PackedSplit: work items one workgroup handles at most
+  int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4 or 8
+  int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
+  int maxItemsPerBlock = 4;  // Packed/PackedSplit: work items one workgroup handles at most
   int mbarOrder = 1;        // order of the Mbar ranks: 0 = input order, 1 = output order
   bool xcdAware = true;     // give every XCD (private L2) a contiguous chunk of the workgroup sequence
 };
@@ -137,6 +139,10 @@ struct PlannerOptions {
 // (reference src/cuttplan.cpp:681-698).  Returns false on an internal error.
 bool createPlans(const Problem& orig, const Problem& red, const cuttHipDeviceProps& props,
                  const PlannerOptions& opt, std::vector<Plan>& plans);
+
+// Same index sets as `src`, launch geometry recomputed under different options (used by the
+// measuring planner to try ordering and granularity variants of its best candidate).
+bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const PlannerOptions& opt, Plan& out);
 
 // Default device description of one MI355X, used when no GPU is present (tests, offline planning).
 cuttHipDeviceProps defaultMI355XProps();

@@ -66,10 +66,12 @@ void cuttSetMethodOverride(int method);
 int cuttGetMethodOverride(void);
 
 /*
- * After cuttPlanMeasure: the candidates it timed, best first is NOT implied;
- * they are in enumeration order.  Returns the number of candidates of the most
- * recent cuttPlanMeasure call of this process and copies up to maxInfos
- * descriptions.
+ * After cuttPlanMeasure: the candidates of its most recent call in this
+ * process, in enumeration order (a variant of the winner that beat it is
+ * appended at the end).  usMeasured is 0 for candidates that were not timed
+ * because the cost model put them more than 1.6x behind its best one
+ * (CUTT_MEASURE_ALL=1 times all).  Returns the number of candidates and copies
+ * up to maxInfos descriptions.
  */
 int cuttGetLastMeasurement(cuttPlanInfo* infos, int maxInfos);
 
