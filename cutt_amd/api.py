@@ -49,6 +49,7 @@ class PlanInfo(ctypes.Structure):
         ("wrSectors", ctypes.c_double), ("ldsCycles", ctypes.c_double), ("blocksPerCU", ctypes.c_double),
         ("usMeasured", ctypes.c_double),
         ("numCandidates", ctypes.c_int), ("planMs", ctypes.c_double),
+        ("cachePolicy", ctypes.c_int), ("elemsPerThread", ctypes.c_int),
     ]
 
     @property
@@ -66,7 +67,8 @@ _lib = None
 
 
 def lib_path():
-    return os.path.join(_HERE, "libcutt.so")
+    """The in-tree build; CUTT_AMD_LIB names another build of the same library (experiments)."""
+    return os.environ.get("CUTT_AMD_LIB") or os.path.join(_HERE, "libcutt.so")
 
 
 def lib():

@@ -127,6 +127,34 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.wrSectors = p.model.wrSectors;
   o.ldsCycles = p.model.ldsCycles;
   o.blocksPerCU = p.model.blocksPerCU;
+  o.cachePolicy = p.method == kTiled ? p.tiled.cachePolicy
+                                      : (p.method == kTiledCopy ? p.tcopy.cachePolicy : p.packed.cachePolicy);
+  o.elemsPerThread = p.packed.elemsPerThread;
+}
+
+void setCachePolicy(Plan& p, int policy) {
+  p.tiled.cachePolicy = policy;
+  p.tcopy.cachePolicy = policy;
+  p.packed.cachePolicy = policy;
+}
+
+int cachePolicyOf(const Plan& p) {
+  if (p.method == kTiled) return p.tiled.cachePolicy;
+  if (p.method == kTiledCopy) return p.tcopy.cachePolicy;
+  return p.packed.cachePolicy;
+}
+
+// Cache policy from the model's sampled address stream.  Streaming loads give up the L2 copy of a
+// line, so they pay off only when a workgroup uses (nearly) whole lines of what it reads;
+// streaming stores only when no written line is left partly covered by a workgroup.
+// (Not applied when CUTT_CACHE_POLICY pins the policy.)
+void chooseCachePolicy(Plan& p) {
+  if (std::getenv("CUTT_CACHE_POLICY")) return;
+  if (p.method == kTrivial) return;
+  const double lines = (double)p.pb.volume * p.pb.elemSize / 128.0;
+  const bool wholeReads = p.model.rdLines <= 1.15 * lines;
+  const bool wholeWrites = p.model.wrPartialLines == 0.0;
+  setCachePolicy(p, wholeReads ? (wholeWrites ? 3 : 1) : 0);
 }
 
 // Index of the candidate with the smallest predicted time; Trivial always wins and ties go to
@@ -152,6 +180,10 @@ PlannerOptions plannerOptions(int forceMethod) {
   }
   if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
   if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_CACHE_POLICY")) {
+    const int v = std::atoi(e);
+    if (v == 0 || v == 1 || v == 3) opt.cachePolicy = v;
+  }
   if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
   if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));
@@ -214,6 +246,7 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
   const int best = chooseHeuristic(plans);
   if (best < 0) return CUTT_INTERNAL_ERROR;
+  chooseCachePolicy(plans[best]);
   return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
 }
 
@@ -236,8 +269,10 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   std::vector<Plan> plans;
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
   if (plans.empty()) return CUTT_INTERNAL_ERROR;
-  for (Plan& p : plans)
+  for (Plan& p : plans) {
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
+    chooseCachePolicy(p);
+  }
 
   size_t numBytes = sizeofType;
   for (int i = 0; i < rank; i++) numBytes *= (size_t)dim[i];
@@ -314,10 +349,22 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
         variants.push_back(v);
       }
     }
+    // ... and the other cache policies of the global accesses
+    const int curPolicy = cachePolicyOf(plans[best]);
+    for (int pol : {0, 1, 3}) {
+      if (pol == curPolicy || std::getenv("CUTT_CACHE_POLICY")) continue;
+      PlannerOptions v = base;
+      v.cachePolicy = pol;
+      v.policyOnly = true;
+      variants.push_back(v);
+    }
     for (const PlannerOptions& v : variants) {
       Plan q;
       if (!rebuildPlan(plans[best], props, v, q)) continue;
-      if (q.numBlocks == plans[best].numBlocks && q.method != kTiled && q.method != kTiledCopy) continue;
+      if (!v.policyOnly) {
+        if (q.numBlocks == plans[best].numBlocks && q.method != kTiled && q.method != kTiledCopy) continue;
+        setCachePolicy(q, curPolicy);
+      }
       if (!estimatePlan(q, props, 10)) continue;
       double t;
       if (!timePlan(q, t)) { failed = true; break; }

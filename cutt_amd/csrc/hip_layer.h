@@ -80,6 +80,7 @@ typedef struct cuttHipTiledArgs {
   uint32_t xcdChunk;  /* 0: workgroup b is logical position b; else (b % 8)*xcdChunk + b/8, and the
                          grid has 8*xcdChunk workgroups */
   uint32_t superM, superK;
+  int cachePolicy;    /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
   cuttHipMbar mbar;
 } cuttHipTiledArgs;
 
@@ -98,6 +99,7 @@ typedef struct cuttHipTiledCopyArgs {
   int order;
   uint32_t xcdChunk;
   uint32_t superM, superK;
+  int cachePolicy;
   cuttHipMbar mbar;
 } cuttHipTiledCopyArgs;
 
@@ -146,6 +148,7 @@ typedef struct cuttHipPackedArgs {
   int maxVol;          /* largest class volume */
   uint32_t xcdChunk;   /* 0: workgroup b is logical block b; else logical block = (b % 8)*xcdChunk + b/8
                           and the grid has 8*xcdChunk workgroups */
+  int cachePolicy;     /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
   cuttHipPackedClass cls[4];
   cuttHipMbar mbar;
 } cuttHipPackedArgs;

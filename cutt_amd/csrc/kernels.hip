@@ -33,6 +33,21 @@
 
 namespace {
 
+// Cache policy of the global accesses, a kernel template parameter NT: bit 0 = non-temporal
+// (streaming) loads, bit 1 = non-temporal stores.  The input is read once, so streaming loads keep
+// the L2 free for the output lines that neighbouring workgroups still have to complete; streaming
+// stores pay off only when every written run covers whole 128-byte lines.
+template <int NT, typename T>
+__device__ __forceinline__ T ldg(const T* p) {
+  if constexpr (NT & 1) return __builtin_nontemporal_load(p);
+  else return *p;
+}
+template <int NT, typename T>
+__device__ __forceinline__ void stg(T* p, T v) {
+  if constexpr (NT & 2) __builtin_nontemporal_store(v, p);
+  else *p = v;
+}
+
 constexpr int kTile = 64;             // tile edge in elements
 constexpr int kTileThreads = 256;     // 4 wavefronts
 constexpr int kTileRows = kTile * kTile / kTileThreads;  // rows per lane: 16
@@ -113,7 +128,7 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
 // ---------------------------------------------------------------------------
 // Tiled: 64x64 tile through padded LDS.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int NT>
 __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledArgs a,
                                                             const T* __restrict__ in,
                                                             T* __restrict__ out) {
@@ -143,7 +158,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
       const uint32_t r = min(wave + kWaves * j, wK);
-      v[j] = src[(k0 + r) * a.strideInK];
+      v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
     }
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
@@ -165,7 +180,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
 #pragma unroll
     for (int j = 0; j < kTileRows; j++) {
       const uint32_t r = min(wave + kWaves * j, wM);
-      dst[(m0 + r) * a.strideOutM] = v[j];
+      stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
     }
   }
 }
@@ -173,7 +188,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
 // ---------------------------------------------------------------------------
 // TiledCopy: rank 0 stays in front; rows are copied through registers.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, int NT>
 __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTiledCopyArgs a,
                                                                 const T* __restrict__ in,
                                                                 T* __restrict__ out) {
@@ -195,12 +210,12 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
 #pragma unroll
   for (int j = 0; j < kTileRows; j++) {
     const uint32_t r = min(wave + kWaves * j, wK);
-    v[j] = src[(k0 + r) * a.strideInK];
+    v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
   }
 #pragma unroll
   for (int j = 0; j < kTileRows; j++) {
     const uint32_t r = min(wave + kWaves * j, wK);
-    dst[(k0 + r) * a.strideOutK] = v[j];
+    stg<NT>(dst + (k0 + r) * a.strideOutK, v[j]);
   }
 }
 
@@ -210,7 +225,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
 
 // E = elements per lane.  Every lane keeps its E table entries in registers, so that the loop
 // over work items does no index arithmetic beyond adding the item's base offsets.
-template <typename T, int E>
+template <typename T, int E, int NT>
 __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
                              T* __restrict__ out) {
   extern __shared__ __align__(16) unsigned char ldsRaw[];
@@ -268,7 +283,7 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
 
     T v[E];
 #pragma unroll
-    for (int j = 0; j < E; j++) v[j] = src[inOff[j]];
+    for (int j = 0; j < E; j++) v[j] = ldg<NT>(src + inOff[j]);
     __syncthreads();  // the previous item has finished reading the LDS buffer
 #pragma unroll
     for (int j = 0; j < E; j++) buf[ldsSlot[j]] = v[j];
@@ -276,7 +291,7 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
 #pragma unroll
     for (int j = 0; j < E; j++) v[j] = buf[shSlot[j]];
 #pragma unroll
-    for (int j = 0; j < E; j++) dst[outOff[j]] = v[j];
+    for (int j = 0; j < E; j++) stg<NT>(dst + outOff[j], v[j]);
   }
 }
 
@@ -329,13 +344,24 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
     return (int)hipErrorInvalidConfiguration;
+  if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
-  if (a->elemSize == 4)
-    hipLaunchKernelGGL(tiledKernel<uint32_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
-                       (const uint32_t*)in, (uint32_t*)out);
-  else
-    hipLaunchKernelGGL(tiledKernel<uint64_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
-                       (const uint64_t*)in, (uint64_t*)out);
+  const dim3 grid((uint32_t)blocks), block(kTileThreads);
+#define CUTT_LAUNCH_TILED(T, NT) \
+  hipLaunchKernelGGL((tiledKernel<T, NT>), grid, block, 0, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_TILED_NT(T)                                \
+  switch (a->cachePolicy) {                                    \
+    case 0: CUTT_LAUNCH_TILED(T, 0); break;                    \
+    case 1: CUTT_LAUNCH_TILED(T, 1); break;                    \
+    default: CUTT_LAUNCH_TILED(T, 3); break;                   \
+  }
+  if (a->elemSize == 4) {
+    CUTT_LAUNCH_TILED_NT(uint32_t)
+  } else {
+    CUTT_LAUNCH_TILED_NT(uint64_t)
+  }
+#undef CUTT_LAUNCH_TILED_NT
+#undef CUTT_LAUNCH_TILED
   return (int)hipGetLastError();
 }
 
@@ -349,13 +375,24 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
     return (int)hipErrorInvalidConfiguration;
+  if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
-  if (a->elemSize == 4)
-    hipLaunchKernelGGL(tiledCopyKernel<uint32_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
-                       (const uint32_t*)in, (uint32_t*)out);
-  else
-    hipLaunchKernelGGL(tiledCopyKernel<uint64_t>, dim3((uint32_t)blocks), dim3(kTileThreads), 0, s, *a,
-                       (const uint64_t*)in, (uint64_t*)out);
+  const dim3 grid((uint32_t)blocks), block(kTileThreads);
+#define CUTT_LAUNCH_TCOPY(T, NT) \
+  hipLaunchKernelGGL((tiledCopyKernel<T, NT>), grid, block, 0, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_TCOPY_NT(T)                                \
+  switch (a->cachePolicy) {                                    \
+    case 0: CUTT_LAUNCH_TCOPY(T, 0); break;                    \
+    case 1: CUTT_LAUNCH_TCOPY(T, 1); break;                    \
+    default: CUTT_LAUNCH_TCOPY(T, 3); break;                   \
+  }
+  if (a->elemSize == 4) {
+    CUTT_LAUNCH_TCOPY_NT(uint32_t)
+  } else {
+    CUTT_LAUNCH_TCOPY_NT(uint64_t)
+  }
+#undef CUTT_LAUNCH_TCOPY_NT
+#undef CUTT_LAUNCH_TCOPY
   return (int)hipGetLastError();
 }
 
@@ -365,6 +402,7 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
       (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
       (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
        a->elemsPerThread != 8) ||
+      (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) ||
       a->padShift > 31 || a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t items = (uint64_t)a->volMbar;
@@ -403,7 +441,10 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     if (e != hipSuccess) return (int)e;
     const size_t m = prop.sharedMemPerBlock;
     int r = 0;
-#define CUTT_ALLOW(T, E) if (r == 0) r = allowLargeLds(packedKernel<T, E>, m)
+#define CUTT_ALLOW(T, E)                                                  \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0>, m);                \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1>, m);                \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3>, m)
     CUTT_ALLOW(uint32_t, 1); CUTT_ALLOW(uint32_t, 2); CUTT_ALLOW(uint32_t, 4); CUTT_ALLOW(uint32_t, 8);
     CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
 #undef CUTT_ALLOW
@@ -412,20 +453,27 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   }
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(a->numThreads);
-#define CUTT_LAUNCH_PACKED(T, E) \
-  hipLaunchKernelGGL((packedKernel<T, E>), grid, block, lds, s, *a, (const T*)in, (T*)out)
-#define CUTT_LAUNCH_PACKED_E(T)                        \
-  switch (a->elemsPerThread) {                         \
-    case 1: CUTT_LAUNCH_PACKED(T, 1); break;           \
-    case 2: CUTT_LAUNCH_PACKED(T, 2); break;           \
-    case 4: CUTT_LAUNCH_PACKED(T, 4); break;           \
-    default: CUTT_LAUNCH_PACKED(T, 8); break;          \
+#define CUTT_LAUNCH_PACKED(T, E, NT) \
+  hipLaunchKernelGGL((packedKernel<T, E, NT>), grid, block, lds, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_PACKED_NT(T, E)                            \
+  switch (a->cachePolicy) {                                    \
+    case 0: CUTT_LAUNCH_PACKED(T, E, 0); break;                \
+    case 1: CUTT_LAUNCH_PACKED(T, E, 1); break;                \
+    default: CUTT_LAUNCH_PACKED(T, E, 3); break;               \
+  }
+#define CUTT_LAUNCH_PACKED_E(T)                                \
+  switch (a->elemsPerThread) {                                 \
+    case 1: CUTT_LAUNCH_PACKED_NT(T, 1) break;                 \
+    case 2: CUTT_LAUNCH_PACKED_NT(T, 2) break;                 \
+    case 4: CUTT_LAUNCH_PACKED_NT(T, 4) break;                 \
+    default: CUTT_LAUNCH_PACKED_NT(T, 8) break;                \
   }
   if (a->elemSize == 4) {
     CUTT_LAUNCH_PACKED_E(uint32_t)
   } else {
     CUTT_LAUNCH_PACKED_E(uint64_t)
   }
+#undef CUTT_LAUNCH_PACKED_NT
 #undef CUTT_LAUNCH_PACKED_E
 #undef CUTT_LAUNCH_PACKED
   return (int)hipGetLastError();

@@ -293,7 +293,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   // --- time estimate ---
   // The estimate is "time of a same-size device-to-device copy" times an overhead factor that is
   // linear in a few transaction ratios.  The coefficients are a least-squares fit to the measured
-  // times of about 2600 candidates over 84 tensors of ~2e8 elements on one MI355X (ranks 2-7, 4- and
+  // times of about 2400 candidates over 84 tensors of ~2e8 elements on one MI355X (ranks 2-7, 4- and
   // 8-byte elements, timed by cuttPlanMeasure); on tensors left out of the fit the plan chosen by
   // this estimate was on average 2 % and at worst 14 % slower than the measured best.
   //  - Tiled / TiledCopy: workgroups on one XCD walk neighbouring tiles, so partly used lines are
@@ -313,10 +313,10 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double tilesM = copy ? plan.tcopy.tilesM : plan.tiled.tilesM;
     const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
     const double waste = tilesM * tilesK * (double)plan.split.volMbar * kTile * kTile / (double)plan.pb.volume - 1.0;
-    factor = 1.03 + 0.30 * waste + (es == 4 ? 0.05 : 0.0) + (copy ? 0.15 : 0.0);
+    factor = 1.00 + 0.30 * waste + (es == 4 ? 0.05 : 0.0) + (copy ? 0.30 : 0.0);
   } else {
-    factor = 1.143 + 0.09 * (rdAmp - 1.0) + 0.22 * (wrAmp - 1.0) + 0.016 * partial + (es == 4 ? 0.04 : 0.0) -
-             (plan.method == kPacked ? 0.066 : 0.0);
+    factor = 1.127 + 0.093 * (rdAmp - 1.0) + 0.223 * (wrAmp - 1.0) + 0.017 * partial + (es == 4 ? 0.038 : 0.0) -
+             (plan.method == kPacked ? 0.072 : 0.0);
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);

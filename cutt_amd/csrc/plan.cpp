@@ -318,6 +318,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   a.elemSize = pb.elemSize;
   a.volMbar = (int)sp.volMbar;
   a.padShift = kPadShift;
+  a.cachePolicy = opt.cachePolicy;
   for (int i = 0; i < 2; i++) {
     cuttHipSplitRank& sr = a.split[i];
     sr.numSplit = 1;
@@ -425,6 +426,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
+    a.cachePolicy = opt.cachePolicy;
     fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
     plan.ldsBytes = (size_t)kTile * (kTile + 1) * pb.elemSize;
   } else {
@@ -442,6 +444,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
+    a.cachePolicy = opt.cachePolicy;
     fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
     plan.ldsBytes = 0;
   }

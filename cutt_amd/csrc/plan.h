@@ -131,6 +131,8 @@ struct PlannerOptions {
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4 or 8
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
   int maxItemsPerBlock = 4;  // Packed/PackedSplit: work items one workgroup handles at most
+  bool policyOnly = false;  // (measuring planner) this variant differs only in the cache policy
+  int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores
   int mbarOrder = 1;        // order of the Mbar ranks: 0 = input order, 1 = output order
   bool xcdAware = true;     // give every XCD (private L2) a contiguous chunk of the workgroup sequence
 };

@@ -49,6 +49,8 @@ typedef struct cuttPlanInfo {
   /* planning statistics of the call that made the plan */
   int numCandidates;
   double planMs;
+  int cachePolicy;      /* 0 default, 1 non-temporal loads, 3 non-temporal loads and stores */
+  int elemsPerThread;   /* Packed/PackedSplit */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */
