@@ -1,4 +1,4 @@
-"""Compile libcutt.so for gfx950 with the committed Makefile (hipcc + g++)."""
+"""Compile libcutt.so and the native drivers for gfx950 with the committed Makefiles (hipcc + g++)."""
 import os
 import subprocess
 
@@ -13,4 +13,12 @@ def build(clean=True, jobs=8):
     path = os.path.join(_HERE, "libcutt.so")
     if not os.path.exists(path):
         raise RuntimeError("build did not produce %s" % path)
+    # native drivers (cutt_test, cutt_bench) link against the library just built
+    drivers = os.path.join(_HERE, "drivers")
+    if clean:
+        subprocess.check_call(["make", "-s", "-C", drivers, "clean"])
+    subprocess.check_call(["make", "-s", "-C", drivers, "-j%d" % jobs])
+    for name in ("cutt_test", "cutt_bench"):
+        if not os.path.exists(os.path.join(_HERE, "bin", name)):
+            raise RuntimeError("build did not produce bin/%s" % name)
     return path

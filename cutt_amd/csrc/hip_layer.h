@@ -54,12 +54,37 @@ typedef struct cuttHipMbarDim {
   uint32_t extent;
   uint32_t strideIn;
   uint32_t strideOut;
+  /* Division constants, filled by cuttHipFinishMbar: the index along this rank is
+   * (m / below) % extent, where `below` is the product of the extents before it; both divisions
+   * are multiply-high + shift (see cuttHipDivisor). */
+  uint32_t belowMul, extentMul;
+  uint32_t ctl; /* belowShift | extentShift << 8 | belowAdd << 16 | extentAdd << 17 */
 } cuttHipMbarDim;
 
 typedef struct cuttHipMbar {
   int n;
   cuttHipMbarDim d[CUTT_MAX_RANK];
 } cuttHipMbar;
+
+/*
+ * Division of a 31-bit number by an invariant divisor d >= 1 without a divide instruction:
+ *   n / d == (mulhi32(n, mul) + n * add) >> shift      for every 0 <= n < 2^31.
+ * For d >= 2: shift = ceil(log2 d) - 1, mul = ceil(2^(32+shift) / d) (fits 32 bits), add = 0;
+ * the rounding error of mul is below d <= 2^(shift+1), so n * error < 2^(32+shift) and the
+ * quotient is exact.  d == 1 is mul = 0, add = 1, shift = 0.
+ */
+typedef struct cuttHipDivisor {
+  uint32_t mul;
+  uint32_t shift;
+  uint32_t add;
+} cuttHipDivisor;
+
+cuttHipDivisor cuttHipMakeDivisor(uint32_t d);
+/* Host evaluation of the formula above (what the kernels compute). */
+uint32_t cuttHipDivide(uint32_t n, cuttHipDivisor dv);
+/* Fill the division constants of an Mbar table whose extents are set.  Returns 0, or -1 if the
+ * product of the extents does not fit 31 bits. */
+int cuttHipFinishMbar(cuttHipMbar* mb);
 
 /*
  * Tiled method: a batch of 2-D transposes between input rank 0 (extent volMm,
@@ -126,6 +151,7 @@ typedef struct cuttHipSplitRank {
   int numSplit;
   int slabFloor, slabRem;
   uint32_t strideIn, strideOut; /* global strides of the rank */
+  cuttHipDivisor div;           /* division by numSplit (cuttHipMakeDivisor) */
 } cuttHipSplitRank;
 
 /*

@@ -30,6 +30,9 @@
 #include <hip/hip_runtime.h>
 
 #include "hip_layer.h"
+#include "mbar_decode.h"
+
+using namespace cutt;
 
 namespace {
 
@@ -52,22 +55,6 @@ constexpr int kTile = 64;             // tile edge in elements
 constexpr int kTileThreads = 256;     // 4 wavefronts
 constexpr int kTileRows = kTile * kTile / kTileThreads;  // rows per lane: 16
 constexpr int kWaves = kTileThreads / 64;
-
-// Decompose Mbar position m (wave-uniform) into input and output offsets.
-__device__ __forceinline__ void mbarOffsets(const cuttHipMbar& mb, uint32_t m, uint32_t& offIn,
-                                            uint32_t& offOut) {
-  uint32_t oi = 0, oo = 0;
-  for (int k = 0; k < mb.n; k++) {
-    const uint32_t e = mb.d[k].extent;
-    const uint32_t q = m / e;
-    const uint32_t i = m - q * e;
-    oi += i * mb.d[k].strideIn;
-    oo += i * mb.d[k].strideOut;
-    m = q;
-  }
-  offIn = oi;
-  offOut = oo;
-}
 
 // Workgroup index -> (tile along Mm, tile along Mk, Mbar position).  Returns false for the
 // padding workgroups of order 3.
@@ -137,7 +124,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
   uint32_t tm, tk, m;
   if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
-  mbarOffsets(a.mbar, m, offIn, offOut);
+  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -195,7 +182,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
   uint32_t tm, tk, m;
   if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
-  mbarOffsets(a.mbar, m, offIn, offOut);
+  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -249,17 +236,19 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // out back to back.
   uint32_t inOff[E], outOff[E], shSlot[E], ldsSlot[E];
   int loaded = -1;
+  const MbarLane mbarLane = loadMbarLane(a.mbar, tid & 63);
+  const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
   for (uint32_t w = w0; w < w1; w++) {
-    const uint32_t t = w / ns0;
+    const uint32_t t = fastDivide(w, div0.mul, div0.shift, div0.add);
     const uint32_t s0 = w - t * ns0;
-    const uint32_t m = t / ns1;
+    const uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
     const uint32_t s1 = t - m * ns1;
     const int c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
     const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
     const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
 
     uint32_t offIn, offOut;
-    mbarOffsets(a.mbar, m, offIn, offOut);
+    mbarOffsets(mbarLane, m, offIn, offOut);
     offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
     offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
 
@@ -300,11 +289,20 @@ size_t packedLdsBytes(const cuttHipPackedArgs* a) {
   return (b + 15) & ~(size_t)15;
 }
 
+// The table must carry the division constants cuttHipFinishMbar derives from its extents.
 bool mbarOk(const cuttHipMbar& mb) {
-  if (mb.n < 0 || mb.n > CUTT_MAX_RANK) return false;
-  for (int k = 0; k < mb.n; k++)
-    if (mb.d[k].extent == 0) return false;
+  cuttHipMbar want = mb;
+  if (cuttHipFinishMbar(&want) != 0) return false;
+  for (int k = 0; k < CUTT_MAX_RANK; k++)
+    if (want.d[k].belowMul != mb.d[k].belowMul || want.d[k].extentMul != mb.d[k].extentMul ||
+        want.d[k].ctl != mb.d[k].ctl)
+      return false;
   return true;
+}
+
+bool divisorOk(const cuttHipDivisor& dv, uint32_t d) {
+  const cuttHipDivisor want = cuttHipMakeDivisor(d);
+  return dv.mul == want.mul && dv.shift == want.shift && dv.add == want.add;
 }
 
 // Number of workgroups of a tiled launch; checks the ordering parameters.
@@ -408,7 +406,8 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   uint64_t items = (uint64_t)a->volMbar;
   for (int i = 0; i < 2; i++) {
     const cuttHipSplitRank& sr = a->split[i];
-    if (sr.numSplit < 1 || sr.slabRem < 0 || sr.slabRem >= sr.numSplit || sr.slabFloor < 0)
+    if (sr.numSplit < 1 || sr.slabRem < 0 || sr.slabRem >= sr.numSplit || sr.slabFloor < 0 ||
+        !divisorOk(sr.div, (uint32_t)sr.numSplit))
       return (int)hipErrorInvalidValue;
     items *= (uint64_t)sr.numSplit;
     if (items > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;

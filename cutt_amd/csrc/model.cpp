@@ -321,7 +321,15 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);
   }
-  const double t = tCopy * factor;
+  double t = tCopy * factor;
+  if (plan.method == kPacked || plan.method == kPackedSplit) {
+    // A workgroup spends about 1.3 us per work item regardless of the item's size (load latency,
+    // two barriers, store issue); with small items that, not bandwidth, sets the time:
+    // items * 1.3 us spread over the resident workgroups of all CUs.
+    const double items = (double)plan.packed.volMbar * plan.packed.split[0].numSplit * plan.packed.split[1].numSplit;
+    const double tItems = items * 1.3e-6 / ((double)props.cuCount * blocksPerCU);
+    t = std::sqrt(t * t + tItems * tItems);
+  }
   r.usPredicted = t * 1e6;
   return true;
 }

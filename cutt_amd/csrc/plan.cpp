@@ -257,6 +257,7 @@ void fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, 
     n++;
   }
   mb.n = n;
+  cuttHipFinishMbar(&mb);  // cannot fail: the extents multiply to at most the tensor's volume < 2^31
 }
 
 // Extent of rank r inside one staged block whose split ranks have the slab sizes slab[0..1].
@@ -330,6 +331,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
       sr.strideOut = (uint32_t)pb.strideOut[sp.splitRank[i]];
       if (sr.slabFloor < 1) return false;
     }
+    sr.div = cuttHipMakeDivisor((uint32_t)sr.numSplit);
   }
   for (int c = 0; c < 4; c++) {
     if (!classUsed(a, c)) continue;

@@ -1,0 +1,65 @@
+"""The native drivers (cutt_test, cutt_bench) built beside the library.
+
+On a machine without a GPU only their command lines are exercised (usage
+paths return before any HIP call); on the GPU a shortened cutt_test and one
+cutt_bench tensor run for real.
+"""
+import os
+import subprocess
+
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+BIN = os.path.join(HERE, "..", "cutt_amd", "bin")
+
+
+def run(name, *args, timeout=300):
+    exe = os.path.join(BIN, name)
+    if not os.path.exists(exe):
+        pytest.fail("%s is not built; run __graft_entry__.build()" % exe)
+    return subprocess.run([exe, *args], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=timeout)
+
+
+def test_usage_without_gpu():
+    r = run("cutt_bench")
+    assert r.returncode == 1 and "-bench benchID" in r.stdout and "-measure" in r.stdout
+    r = run("cutt_bench", "-elemsize", "3", "-bench", "6")
+    assert r.returncode == 1
+    r = run("cutt_bench", "-dim", "4", "5", "-permutation", "1")
+    assert r.returncode == 1
+    r = run("cutt_test", "-nonsense")
+    assert r.returncode == 1 and "-device gpuid" in r.stdout
+
+
+@pytest.mark.gpu
+def test_cutt_test_short_run():
+    # all six groups; group 2 with 5 random tensors per rank instead of 100
+    r = run("cutt_test", "-samples", "5", "-seed", "3", timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "test OK" in r.stdout
+    for k in range(1, 7):
+        assert "test %d passed" % k in r.stdout
+
+
+@pytest.mark.gpu
+def test_cutt_test_with_measuring_planner():
+    r = run("cutt_test", "-tests", "3,4,6", "-measure", timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "test OK" in r.stdout
+
+
+@pytest.mark.gpu
+def test_cutt_bench_single_tensor_and_memcpy():
+    r = run("cutt_bench", "-dim", "1024", "64", "1024", "3", "-permutation", "2", "1", "0", "3", "-plantimer")
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout and "method Tiled" in r.stdout and "plan took" in r.stdout
+    r = run("cutt_bench", "-memcpy", "50000000", "-elemsize", "4")
+    assert r.returncode == 0 and "bench OK" in r.stdout and "hipMemcpyDtoD average" in r.stdout
+
+
+@pytest.mark.gpu
+def test_cutt_bench_ttc_suite():
+    r = run("cutt_bench", "-bench", "6", "-nomemcpy", timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout
+    assert r.stdout.count("number of elements") == 57
