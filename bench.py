@@ -30,8 +30,8 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 # HBM bytes per launch of the C2 transpose kernel from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE
 # in runs of their own, each scaled by what the counter reads for the same-size device-to-device
-# copy): 1 610 694 656 fetched + 1 610 612 736 written.  Only valid for the Tiled plan of C2.
-C2_TILED_TRAFFIC_BYTES = 3221307392
+# copy): 1 610 695 680 fetched + 1 611 192 627 written.  Only valid for the Tiled plan of C2.
+C2_TILED_TRAFFIC_BYTES = 3221888307
 
 
 def log(*a):

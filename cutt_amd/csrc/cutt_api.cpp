@@ -579,11 +579,11 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
     } break;
     case 4:
       if (!packed) return -1;
-      v.assign(p.tab[cls].inOff.begin(), p.tab[cls].inOff.end());
+      v.assign(p.tab[cls].rowIn.begin(), p.tab[cls].rowIn.end());
       break;
     case 5:
       if (!packed) return -1;
-      v.assign(p.tab[cls].outOff.begin(), p.tab[cls].outOff.end());
+      v.assign(p.tab[cls].rowOut.begin(), p.tab[cls].rowOut.end());
       break;
     case 6:
       if (!packed) return -1;

@@ -129,19 +129,23 @@ typedef struct cuttHipTiledCopyArgs {
 } cuttHipTiledCopyArgs;
 
 /*
- * Index-remap tables of a Packed / PackedSplit plan for one slab-size class (device pointers,
- * `vol` entries each).  The staged block holds `vol` elements.  Element p in input-compact
- * order is read from input offset inOff[p] and parked in LDS slot p + (p >> padShift).
- * Element q in output-compact order is written to output offset outOff[q] and taken from LDS
- * slot shIdx[q] (padding included).  A workgroup reads its slice of the tables once and keeps
- * it in registers for all the work items it handles.
+ * Index-remap tables of a Packed / PackedSplit plan for one slab-size class (device pointers).
+ * The staged block holds `vol` elements.  In input-compact order the block is vol/inCont
+ * contiguous runs of inCont elements: element p is read from input offset
+ * rowIn[p / inCont] + p % inCont and parked in LDS slot p + (p >> padShift).  In output-compact
+ * order it is vol/outCont runs of outCont elements: element q is written to output offset
+ * rowOut[q / outCont] + q % outCont and taken from LDS slot shIdx[q] (padding included).
+ * A workgroup derives its lanes' offsets once and keeps them in registers for all the work
+ * items it handles; one offset per run instead of one per element keeps the tables small
+ * (2 bytes per element plus 4 per run), since every workgroup reads them through the L2.
  */
 typedef struct cuttHipPackedClass {
   int vol;
-  int inCont, outCont;       /* contiguous run lengths (informational) */
-  const uint32_t* inOff;
-  const uint32_t* outOff;
-  const uint16_t* shIdx;
+  int inCont, outCont;       /* contiguous run lengths; both divide vol */
+  cuttHipDivisor inDiv, outDiv; /* divisions by inCont / outCont (cuttHipMakeDivisor) */
+  const uint32_t* rowIn;     /* vol / inCont entries */
+  const uint32_t* rowOut;    /* vol / outCont entries */
+  const uint16_t* shIdx;     /* vol entries */
 } cuttHipPackedClass;
 
 /* One split rank of a PackedSplit plan: the rank is cut into numSplit slabs; slab s covers

@@ -253,15 +253,19 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
     offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
 
     if (c != loaded) {  // wave-uniform: the class changes at most a few times per workgroup
-      const uint32_t last = (uint32_t)a.cls[c].vol - 1;
-      const uint32_t* gIn = a.cls[c].inOff;
-      const uint32_t* gOut = a.cls[c].outOff;
-      const uint16_t* gSh = a.cls[c].shIdx;
+      const cuttHipPackedClass& k = a.cls[c];
+      const uint32_t last = (uint32_t)k.vol - 1;
+      const uint32_t inCont = (uint32_t)k.inCont, outCont = (uint32_t)k.outCont;
+      const uint32_t* gIn = k.rowIn;
+      const uint32_t* gOut = k.rowOut;
+      const uint16_t* gSh = k.shIdx;
 #pragma unroll
       for (int j = 0; j < E; j++) {
         const uint32_t p = min(tid + j * nt, last);
-        inOff[j] = gIn[p];
-        outOff[j] = gOut[p];
+        const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
+        const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
+        inOff[j] = gIn[ri] + (p - ri * inCont);
+        outOff[j] = gOut[ro] + (p - ro * outCont);
         shSlot[j] = gSh[p];
         ldsSlot[j] = p + (p >> padShift);
       }
@@ -416,8 +420,9 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     // class c is used only if the split ranks it refers to have slabs of the larger size
     if (((c & 1) && a->split[0].slabRem == 0) || ((c & 2) && a->split[1].slabRem == 0)) continue;
     const cuttHipPackedClass& k = a->cls[c];
-    if (k.vol < 1 || k.vol > a->maxVol || (int64_t)a->numThreads * a->elemsPerThread < k.vol || !k.inOff ||
-        !k.outOff || !k.shIdx)
+    if (k.vol < 1 || k.vol > a->maxVol || (int64_t)a->numThreads * a->elemsPerThread < k.vol || !k.rowIn ||
+        !k.rowOut || !k.shIdx || k.inCont < 1 || k.outCont < 1 || k.vol % k.inCont || k.vol % k.outCont ||
+        !divisorOk(k.inDiv, (uint32_t)k.inCont) || !divisorOk(k.outDiv, (uint32_t)k.outCont))
       return (int)hipErrorInvalidValue;
     const uint32_t last = (uint32_t)k.vol - 1;
     if ((int)(last + (last >> a->padShift)) >= a->ldsElems) return (int)hipErrorInvalidValue;

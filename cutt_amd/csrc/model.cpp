@@ -275,8 +275,14 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
       offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
       total.add(packedSample(plan, cls, offIn, offOut), (double)items / ns);
     }
-    // Every workgroup loads its tables once from L2.
-    tableBytes = (double)plan.numBlocks * 10.0 * a.maxVol;
+    // Every workgroup loads its tables once from L2: 2 bytes per element and 4 per run.
+    {
+      int big = 0;
+      for (int c = 1; c < 4; c++)
+        if (plan.tab[c].vol > plan.tab[big].vol) big = c;
+      const PackedTables& t = plan.tab[big];
+      tableBytes = (double)plan.numBlocks * (2.0 * t.vol + 4.0 * (double)(t.rowIn.size() + t.rowOut.size()));
+    }
   }
   r.rdLines = total.rdLines; r.wrLines = total.wrLines;
   r.rdInstr = total.rdInstr; r.wrInstr = total.wrInstr;

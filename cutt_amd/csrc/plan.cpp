@@ -209,8 +209,8 @@ void Plan::release() {
     cuttHipFree(dTables);
     dTables = nullptr;
     for (int c = 0; c < 4; c++) {
-      packed.cls[c].inOff = nullptr;
-      packed.cls[c].outOff = nullptr;
+      packed.cls[c].rowIn = nullptr;
+      packed.cls[c].rowOut = nullptr;
       packed.cls[c].shIdx = nullptr;
     }
   }
@@ -343,6 +343,8 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
     k.vol = (int)vol;
     k.inCont = (int)ic;
     k.outCont = (int)oc;
+    k.inDiv = cuttHipMakeDivisor((uint32_t)ic);
+    k.outDiv = cuttHipMakeDivisor((uint32_t)oc);
     a.maxVol = std::max(a.maxVol, k.vol);
   }
   const int64_t slots = paddedSlots(a.maxVol);
@@ -743,13 +745,6 @@ bool Plan::buildTables() {
     enumerateOffsets(gather, t.vol, pos);
     t.shIdx.resize(pos.size());
     for (size_t q = 0; q < pos.size(); q++) t.shIdx[q] = (uint16_t)(pos[q] + (pos[q] >> packed.padShift));
-    // Per-element offsets: row offset + column inside the contiguous run.
-    t.inOff.resize((size_t)t.vol);
-    t.outOff.resize((size_t)t.vol);
-    for (int p = 0; p < t.vol; p++) {
-      t.inOff[(size_t)p] = t.rowIn[(size_t)(p / t.inCont)] + (uint32_t)(p % t.inCont);
-      t.outOff[(size_t)p] = t.rowOut[(size_t)(p / t.outCont)] + (uint32_t)(p % t.outCont);
-    }
   }
   tablesBuilt = true;
   return true;
@@ -759,21 +754,21 @@ int Plan::activate() {
   if (method != kPacked && method != kPackedSplit) return 0;
   if (dTables) return 0;
   if (!buildTables()) return -1;
-  // One allocation: [inOff | outOff | shIdx] per class, each piece 16-byte aligned.
+  // One allocation: [rowIn | rowOut | shIdx] per class, each piece 16-byte aligned.
   auto align16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
   size_t total = 0;
   size_t off[4][3] = {};
   for (int c = 0; c < 4; c++) {
     if (!classUsed(packed, c)) continue;
-    off[c][0] = total; total += align16(tab[c].inOff.size() * sizeof(uint32_t));
-    off[c][1] = total; total += align16(tab[c].outOff.size() * sizeof(uint32_t));
+    off[c][0] = total; total += align16(tab[c].rowIn.size() * sizeof(uint32_t));
+    off[c][1] = total; total += align16(tab[c].rowOut.size() * sizeof(uint32_t));
     off[c][2] = total; total += align16(tab[c].shIdx.size() * sizeof(uint16_t));
   }
   std::vector<unsigned char> host(total, 0);
   for (int c = 0; c < 4; c++) {
     if (!classUsed(packed, c)) continue;
-    std::memcpy(&host[off[c][0]], tab[c].inOff.data(), tab[c].inOff.size() * sizeof(uint32_t));
-    std::memcpy(&host[off[c][1]], tab[c].outOff.data(), tab[c].outOff.size() * sizeof(uint32_t));
+    std::memcpy(&host[off[c][0]], tab[c].rowIn.data(), tab[c].rowIn.size() * sizeof(uint32_t));
+    std::memcpy(&host[off[c][1]], tab[c].rowOut.data(), tab[c].rowOut.size() * sizeof(uint32_t));
     std::memcpy(&host[off[c][2]], tab[c].shIdx.data(), tab[c].shIdx.size() * sizeof(uint16_t));
   }
   void* d = nullptr;
@@ -788,8 +783,8 @@ int Plan::activate() {
   for (int c = 0; c < 4; c++) {
     if (!classUsed(packed, c)) continue;
     unsigned char* base = (unsigned char*)d;
-    packed.cls[c].inOff = (const uint32_t*)(base + off[c][0]);
-    packed.cls[c].outOff = (const uint32_t*)(base + off[c][1]);
+    packed.cls[c].rowIn = (const uint32_t*)(base + off[c][0]);
+    packed.cls[c].rowOut = (const uint32_t*)(base + off[c][1]);
     packed.cls[c].shIdx = (const uint16_t*)(base + off[c][2]);
   }
   return 0;

@@ -67,13 +67,11 @@ struct Split {
   int64_t volStaged() const;  // elements one workgroup stages at most
 };
 
-// Host copy of the index tables of one slab-size class.  rowIn/rowOut hold one offset per
-// contiguous run (the cost model walks those); inOff/outOff/shIdx are the per-element tables the
-// kernel reads (see cuttHipPackedClass).
+// Host copy of the index tables of one slab-size class (see cuttHipPackedClass): one offset per
+// contiguous run on the input and on the output side, and the LDS gather index per element.
 struct PackedTables {
   int vol = 0, inCont = 0, outCont = 0;
   std::vector<uint32_t> rowIn, rowOut;
-  std::vector<uint32_t> inOff, outOff;
   std::vector<uint16_t> shIdx;
 };
 

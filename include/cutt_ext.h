@@ -123,7 +123,8 @@ int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
  *           elemsPerThread, then for each of the two split slots: numSplit, slabFloor, slabRem,
  *           strideIn, strideOut
  *   what 3: class scalars: vol, inCont, outCont
- *   what 4: inOff[]   what 5: outOff[]   what 6: shIdx[]
+ *   what 4: rowIn[] (vol/inCont input offsets, one per contiguous run)
+ *   what 5: rowOut[] (vol/outCont output offsets)   what 6: shIdx[] (vol LDS gather slots)
  */
 long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                              long long maxCount);

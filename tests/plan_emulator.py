@@ -123,10 +123,14 @@ def emulate(cands, idx, data):
         if ((c & 1) and splits[0][2] == 0) or ((c & 2) and splits[1][2] == 0):
             continue
         cvol, in_cont, out_cont = [int(v) for v in cands.data(idx, 3, c)]
-        in_off, out_off, sh = cands.data(idx, 4, c), cands.data(idx, 5, c), cands.data(idx, 6, c)
-        assert len(in_off) == cvol and len(out_off) == cvol and len(sh) == cvol
+        row_in, row_out, sh = cands.data(idx, 4, c), cands.data(idx, 5, c), cands.data(idx, 6, c)
+        assert cvol % in_cont == 0 and cvol % out_cont == 0
+        assert len(row_in) == cvol // in_cont and len(row_out) == cvol // out_cont and len(sh) == cvol
         assert cvol <= num_threads * elems_per_thread, "a lane would need more table registers"
         p = np.arange(cvol, dtype=np.int64)
+        # per-element offsets as the kernel derives them: run offset + position inside the run
+        in_off = row_in[p // in_cont] + p % in_cont
+        out_off = row_out[p // out_cont] + p % out_cont
         slot = p + (p >> pad_shift)
         assert slot.max() < lds_elems, "LDS slot outside the buffer"
         assert len(np.unique(slot)) == cvol
