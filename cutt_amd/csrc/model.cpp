@@ -299,12 +299,13 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   // --- time estimate ---
   // The estimate is "time of a same-size device-to-device copy" times an overhead factor that is
   // linear in a few transaction ratios.  The coefficients are a least-squares fit to the measured
-  // times of about 2400 candidates over 84 tensors of ~2e8 elements on one MI355X (ranks 2-7, 4- and
-  // 8-byte elements, timed by cuttPlanMeasure); on tensors left out of the fit the plan chosen by
-  // this estimate was on average 2 % and at worst 14 % slower than the measured best.
+  // times of about 7700 candidates over 197 tensors of 1e8-2e8 elements on one MI355X (ranks 2-15, 4-
+  // and 8-byte elements, timed by cuttPlanMeasure); over those tensors the plan chosen by this estimate is
+  // on average 6 % (median 3.5 %, worst 39 %) slower than the measured best candidate.
   //  - Tiled / TiledCopy: workgroups on one XCD walk neighbouring tiles, so partly used lines are
-  //    found in the L2 and the line counts hardly matter; what costs is the padding of edge
-  //    tiles, whose clamped lanes repeat accesses that hit the L1 (about a quarter of a real one).
+  //    mostly found in the L2 and extra lines cost less than for the packed kernel; the padding
+  //    of edge tiles, whose clamped lanes repeat accesses that hit the L1, costs about a quarter
+  //    of a real access.
   //  - Packed / PackedSplit: extra lines on the write side cost about twice as much as on the read
   //    side (partly written lines have to be merged in the L2), 4-byte elements a little more per
   //    byte than 8-byte ones, and a block cut into slabs a little more than a whole one.
@@ -319,7 +320,8 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double tilesM = copy ? plan.tcopy.tilesM : plan.tiled.tilesM;
     const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
     const double waste = tilesM * tilesK * (double)plan.split.volMbar * kTile * kTile / (double)plan.pb.volume - 1.0;
-    factor = 1.00 + 0.30 * waste + (es == 4 ? 0.05 : 0.0) + (copy ? 0.30 : 0.0);
+    factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
+             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0);
   } else {
     factor = 1.127 + 0.093 * (rdAmp - 1.0) + 0.223 * (wrAmp - 1.0) + 0.017 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.072 : 0.0);
