@@ -176,7 +176,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_XCD_AWARE")) opt.xcdAware = std::atoi(e) != 0;
   if (const char* e = std::getenv("CUTT_ELEMS_PER_THREAD")) {
     const int v = std::atoi(e);
-    if (v == 1 || v == 2 || v == 4 || v == 8) opt.elemsPerThread = v;
+    if (v == 1 || v == 2 || v == 4 || v == 8 || v == 16) opt.elemsPerThread = v;
   }
   if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
   if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
@@ -184,6 +184,7 @@ PlannerOptions plannerOptions(int forceMethod) {
     const int v = std::atoi(e);
     if (v == 0 || v == 1 || v == 3) opt.cachePolicy = v;
   }
+  if (const char* e = std::getenv("CUTT_WIDE_OFFSETS")) opt.wideOffsets = std::atoi(e) != 0;
   if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
   if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));

@@ -172,19 +172,28 @@ typedef struct cuttHipPackedArgs {
   int volMbar;
   cuttHipSplitRank split[2];
   int itemsPerBlock;
-  int elemsPerThread;  /* 1, 2, 4 or 8: numThreads*elemsPerThread >= vol of every class */
+  int elemsPerThread;  /* 1, 2, 4, 8 or (4-byte elements only) 16: numThreads*elemsPerThread >= vol of every class */
   int padShift;        /* LDS slot(p) = p + (p >> padShift); 31 = no padding */
   int ldsElems;        /* element slots in the LDS data buffer (padding included) */
   int maxVol;          /* largest class volume */
   uint32_t xcdChunk;   /* 0: workgroup b is logical block b; else logical block = (b % 8)*xcdChunk + b/8
                           and the grid has 8*xcdChunk workgroups */
   int cachePolicy;     /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
+  long long volume;    /* elements of the whole tensor (bounds every offset) */
+  int wideOffsets;     /* 0: the tensor is below 4 GB and the kernel keeps 32-bit byte offsets;
+                          1: element offsets with 64-bit address arithmetic (required from 4 GB on) */
   cuttHipPackedClass cls[4];
   cuttHipMbar mbar;
 } cuttHipPackedArgs;
 
 /* Bytes of LDS the packed kernel needs for these arguments. */
 size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a);
+/* Vector registers per lane of the packed kernel instance for this element size, elements per lane
+ * and offset width, as built (a table kept beside the kernel; needs no GPU).  The planner derives
+ * the resident wavefronts per CU from it: min(8, 512 / roundup8(registers)) per SIMD, 4 SIMDs. */
+int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets);
+/* The same number asked of the HIP runtime for the loaded code object (needs a GPU); -1 on error. */
+int cuttHipPackedRegsPerLaneLoaded(int elemSize, int elemsPerThread, int wideOffsets);
 
 /* ---- device, memory, stream and event helpers ---------------------------- */
 int cuttHipGetDevice(int* device);

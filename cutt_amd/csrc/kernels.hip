@@ -212,11 +212,14 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
 
 // E = elements per lane.  Every lane keeps its E table entries in registers, so that the loop
 // over work items does no index arithmetic beyond adding the item's base offsets.
-template <typename T, int E, int NT>
+// WIDE = false: the tensor is smaller than 4 GB, so the lanes keep 32-bit byte offsets and every
+// access is "uniform 64-bit base + 32-bit lane offset" (no per-access 64-bit address registers).  WIDE = true:
+// element offsets and 64-bit address arithmetic.
+template <typename T, int E, int NT, bool WIDE>
 __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
                              T* __restrict__ out) {
   extern __shared__ __align__(16) unsigned char ldsRaw[];
-  T* buf = reinterpret_cast<T*>(ldsRaw);
+  constexpr uint32_t kScale = WIDE ? 1u : (uint32_t)sizeof(T);
 
   const uint32_t tid = threadIdx.x;
   const uint32_t nt = blockDim.x;
@@ -234,7 +237,9 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // Lanes whose element index lies beyond the block repeat the block's last element (same
   // addresses, same value), so that the code below has no branches and every lane's E loads go
   // out back to back.
-  uint32_t inOff[E], outOff[E], shSlot[E], ldsSlot[E];
+  uint32_t inOff[E], outOff[E];  // global offsets: bytes (narrow) or elements (wide)
+  uint32_t shSlot[E];            // byte offset of the LDS slot an output element is taken from
+  uint32_t last = 0;             // last element index of the loaded class
   int loaded = -1;
   const MbarLane mbarLane = loadMbarLane(a.mbar, tid & 63);
   const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
@@ -254,7 +259,7 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
 
     if (c != loaded) {  // wave-uniform: the class changes at most a few times per workgroup
       const cuttHipPackedClass& k = a.cls[c];
-      const uint32_t last = (uint32_t)k.vol - 1;
+      last = (uint32_t)k.vol - 1;
       const uint32_t inCont = (uint32_t)k.inCont, outCont = (uint32_t)k.outCont;
       const uint32_t* gIn = k.rowIn;
       const uint32_t* gOut = k.rowOut;
@@ -264,27 +269,50 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
         const uint32_t p = min(tid + j * nt, last);
         const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
         const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
-        inOff[j] = gIn[ri] + (p - ri * inCont);
-        outOff[j] = gOut[ro] + (p - ro * outCont);
-        shSlot[j] = gSh[p];
-        ldsSlot[j] = p + (p >> padShift);
+        // uniform base + 32-bit lane offset here too (the tables are far smaller than 4 GB)
+        const uint32_t rowI = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gIn) + ri * 4u);
+        const uint32_t rowO = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gOut) + ro * 4u);
+        const uint32_t sh = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const unsigned char*>(gSh) + p * 2u);
+        inOff[j] = (rowI + (p - ri * inCont)) * kScale;
+        outOff[j] = (rowO + (p - ro * outCont)) * kScale;
+        shSlot[j] = sh * (uint32_t)sizeof(T);
       }
       loaded = c;
     }
-    const T* src = in + offIn;
-    T* dst = out + offOut;
+    // wave-uniform bases of this item
+    const unsigned char* srcB = reinterpret_cast<const unsigned char*>(in + offIn);
+    unsigned char* dstB = reinterpret_cast<unsigned char*>(out + offOut);
 
     T v[E];
 #pragma unroll
-    for (int j = 0; j < E; j++) v[j] = ldg<NT>(src + inOff[j]);
+    for (int j = 0; j < E; j++) {
+      if (WIDE)
+        v[j] = ldg<NT>(reinterpret_cast<const T*>(srcB) + inOff[j]);
+      else
+        v[j] = ldg<NT>(reinterpret_cast<const T*>(srcB + inOff[j]));
+    }
     __syncthreads();  // the previous item has finished reading the LDS buffer
+    {
+      // The slot of element p is p + (p >> padShift).  It is recomputed for every item from a
+      // value the compiler cannot see through, so that it does not park E more registers.
+      uint32_t tv = tid;
+      asm volatile("" : "+v"(tv));
 #pragma unroll
-    for (int j = 0; j < E; j++) buf[ldsSlot[j]] = v[j];
+      for (int j = 0; j < E; j++) {
+        const uint32_t p = min(tv + j * nt, last);
+        *reinterpret_cast<T*>(ldsRaw + (p + (p >> padShift)) * (uint32_t)sizeof(T)) = v[j];
+      }
+    }
     __syncthreads();
 #pragma unroll
-    for (int j = 0; j < E; j++) v[j] = buf[shSlot[j]];
+    for (int j = 0; j < E; j++) v[j] = *reinterpret_cast<const T*>(ldsRaw + shSlot[j]);
 #pragma unroll
-    for (int j = 0; j < E; j++) stg<NT>(dst + outOff[j], v[j]);
+    for (int j = 0; j < E; j++) {
+      if (WIDE)
+        stg<NT>(reinterpret_cast<T*>(dstB) + outOff[j], v[j]);
+      else
+        stg<NT>(reinterpret_cast<T*>(dstB + outOff[j]), v[j]);
+    }
   }
 }
 
@@ -336,6 +364,48 @@ int allowLargeLds(K kernel, size_t bytes) {
 }  // namespace
 
 extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) { return packedLdsBytes(a); }
+
+// Registers per lane of packedKernel<T, E, *, WIDE> as compiled for gfx950 (the cache policy does
+// not change the count).  Rows: E = 1, 2, 4, 8, 16.
+extern "C" int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets) {
+  static const int narrow4[5] = {14, 22, 37, 67, 103}, wide4[5] = {17, 27, 47, 69, 128};
+  static const int narrow8[5] = {15, 23, 41, 73, 0}, wide8[5] = {18, 29, 51, 78, 0};
+  int row = 0;
+  while (row < 5 && (1 << row) != elemsPerThread) row++;
+  if (row == 5 || (elemSize != 4 && elemSize != 8)) return 0;
+  return elemSize == 4 ? (wideOffsets ? wide4 : narrow4)[row] : (wideOffsets ? wide8 : narrow8)[row];
+}
+
+extern "C" int cuttHipPackedRegsPerLaneLoaded(int elemSize, int elemsPerThread, int wideOffsets) {
+  const void* f = nullptr;
+#define CUTT_PICK(T, E)                                                                       \
+  f = wideOffsets ? reinterpret_cast<const void*>(packedKernel<T, E, 0, true>)               \
+                  : reinterpret_cast<const void*>(packedKernel<T, E, 0, false>)
+  if (elemSize == 4) {
+    switch (elemsPerThread) {
+      case 1: CUTT_PICK(uint32_t, 1); break;
+      case 2: CUTT_PICK(uint32_t, 2); break;
+      case 4: CUTT_PICK(uint32_t, 4); break;
+      case 8: CUTT_PICK(uint32_t, 8); break;
+      case 16: CUTT_PICK(uint32_t, 16); break;
+      default: return -1;
+    }
+  } else if (elemSize == 8) {
+    switch (elemsPerThread) {
+      case 1: CUTT_PICK(uint64_t, 1); break;
+      case 2: CUTT_PICK(uint64_t, 2); break;
+      case 4: CUTT_PICK(uint64_t, 4); break;
+      case 8: CUTT_PICK(uint64_t, 8); break;
+      default: return -1;
+    }
+  } else {
+    return -1;
+  }
+#undef CUTT_PICK
+  hipFuncAttributes attr;
+  if (hipFuncGetAttributes(&attr, f) != hipSuccess) return -1;
+  return attr.numRegs;
+}
 
 extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, void* out, void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
@@ -403,9 +473,12 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
       (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
       (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
-       a->elemsPerThread != 8) ||
+       a->elemsPerThread != 8 && !(a->elemsPerThread == 16 && a->elemSize == 4)) ||
       (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) ||
-      a->padShift > 31 || a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar))
+      a->padShift > 31 || a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar) || a->volume < 1 ||
+      a->volume > 0x7fffffffll ||
+      // 32-bit byte offsets reach 4 GB
+      (!a->wideOffsets && (uint64_t)a->volume * (uint64_t)a->elemSize > (1ull << 32)))
     return (int)hipErrorInvalidValue;
   uint64_t items = (uint64_t)a->volMbar;
   for (int i = 0; i < 2; i++) {
@@ -446,10 +519,14 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     const size_t m = prop.sharedMemPerBlock;
     int r = 0;
 #define CUTT_ALLOW(T, E)                                                  \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0>, m);                \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1>, m);                \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3>, m)
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, true>, m);          \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, true>, m);          \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, true>, m)
     CUTT_ALLOW(uint32_t, 1); CUTT_ALLOW(uint32_t, 2); CUTT_ALLOW(uint32_t, 4); CUTT_ALLOW(uint32_t, 8);
+    CUTT_ALLOW(uint32_t, 16);
     CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
 #undef CUTT_ALLOW
     if (r != 0) return r;
@@ -457,8 +534,12 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   }
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(a->numThreads);
-#define CUTT_LAUNCH_PACKED(T, E, NT) \
-  hipLaunchKernelGGL((packedKernel<T, E, NT>), grid, block, lds, s, *a, (const T*)in, (T*)out)
+  const bool wide = a->wideOffsets != 0;
+#define CUTT_LAUNCH_PACKED(T, E, NT)                                                                    \
+  if (wide)                                                                                            \
+    hipLaunchKernelGGL((packedKernel<T, E, NT, true>), grid, block, lds, s, *a, (const T*)in, (T*)out); \
+  else                                                                                                 \
+    hipLaunchKernelGGL((packedKernel<T, E, NT, false>), grid, block, lds, s, *a, (const T*)in, (T*)out)
 #define CUTT_LAUNCH_PACKED_NT(T, E)                            \
   switch (a->cachePolicy) {                                    \
     case 0: CUTT_LAUNCH_PACKED(T, E, 0); break;                \
@@ -472,7 +553,10 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     case 4: CUTT_LAUNCH_PACKED_NT(T, 4) break;                 \
     default: CUTT_LAUNCH_PACKED_NT(T, 8) break;                \
   }
-  if (a->elemSize == 4) {
+  if (a->elemSize == 4 && a->elemsPerThread == 16) {
+    // 4-byte elements only: 16 per lane stage the same 64 KB as 8 per lane do for 8-byte elements
+    CUTT_LAUNCH_PACKED_NT(uint32_t, 16)
+  } else if (a->elemSize == 4) {
     CUTT_LAUNCH_PACKED_E(uint32_t)
   } else {
     CUTT_LAUNCH_PACKED_E(uint64_t)

@@ -292,7 +292,13 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
 
   // Resident workgroups per CU.
   const double byLds = plan.ldsBytes ? std::floor((double)props.ldsPerCU / (double)plan.ldsBytes) : 32.0;
-  const double byThreads = std::floor((double)props.maxThreadsPerCU / plan.numThreads);
+  // Wavefronts that fit a CU by registers: 512 per SIMD lane, allocated in units of 8, 4 SIMDs.
+  double threadsByRegs = (double)props.maxThreadsPerCU;
+  if (plan.method == kPacked || plan.method == kPackedSplit) {
+    const int regs = cuttHipPackedRegsPerLane(plan.pb.elemSize, plan.packed.elemsPerThread, plan.packed.wideOffsets);
+    if (regs > 0) threadsByRegs = std::min(threadsByRegs, 4.0 * 64.0 * std::min(8, 512 / ((regs + 7) / 8 * 8)));
+  }
+  const double byThreads = std::floor(threadsByRegs / plan.numThreads);
   const double blocksPerCU = std::max(1.0, std::min({byLds, byThreads, 32.0}));
   r.blocksPerCU = blocksPerCU;
 

@@ -291,23 +291,34 @@ inline bool classUsed(const cuttHipPackedArgs& a, int c) {
   return !((c & 1) && a.split[0].slabRem == 0) && !((c & 2) && a.split[1].slabRem == 0);
 }
 
-// Threads per workgroup and elements per lane (1, 2, 4, 8) for a staged block of `vol`
-// elements.  numThreads = 0: does not fit.  Eight elements per lane is the most the kernel keeps
-// in registers without losing occupancy (three table words and one data word per element).
-constexpr int kMaxElemsPerThread = 8;
+// Threads per workgroup and elements per lane (1, 2, 4, 8, 16) for a staged block of `vol`
+// elements.  numThreads = 0: does not fit.  A lane keeps three table words and the data of each of
+// its elements in registers; 64 bytes of data per lane (8 x 8 bytes or 16 x 4 bytes) is the most
+// that fits 128 registers, the budget of a 1024-lane workgroup.
+inline int maxElemsPerThread(int elemSize) { return elemSize == 4 ? 16 : 8; }
 
-void choosePackedThreads(int64_t vol, const cuttHipDeviceProps& props, int opt_e, int& numThreads,
+void choosePackedThreads(int64_t vol, int elemSize, const cuttHipDeviceProps& props, int opt_e, int& numThreads,
                          int& elemsPerThread) {
+  const int kMaxElemsPerThread = maxElemsPerThread(elemSize);
   numThreads = 0;
   elemsPerThread = 0;
   // As many elements per lane as the block allows: the loads a lane has in flight are what hides
   // the memory latency, and smaller workgroups leave room for more of them on a CU.
-  int e = opt_e > 0 ? opt_e : (vol >= 512 ? 8 : (vol >= 256 ? 4 : (vol > 64 ? 2 : 1)));
+  int e = opt_e > 0 ? std::min(opt_e, kMaxElemsPerThread) : (vol >= 512 ? 8 : (vol >= 256 ? 4 : (vol > 64 ? 2 : 1)));
   while (e < kMaxElemsPerThread && roundUp64(ceilDiv(vol, e)) > props.maxThreadsPerBlock) e *= 2;
   const int64_t nt = roundUp64(ceilDiv(vol, e));
   if (nt > props.maxThreadsPerBlock) return;
   numThreads = (int)nt;
   elemsPerThread = e;
+}
+
+// Lanes of the packed kernel that fit a CU: 512 registers per SIMD lane in units of 8, 4 SIMDs of
+// 64-lane wavefronts, at most 8 wavefronts per SIMD.
+int64_t packedThreadsPerCU(const cuttHipDeviceProps& props, int elemSize, int elemsPerThread, int wide) {
+  const int regs = cuttHipPackedRegsPerLane(elemSize, elemsPerThread, wide);
+  int64_t t = props.maxThreadsPerCU;
+  if (regs > 0) t = std::min<int64_t>(t, 4 * 64 * std::min(8, 512 / ((regs + 7) / 8 * 8)));
+  return t;
 }
 
 // Fill the launch geometry of a Packed / PackedSplit candidate.  False = does not fit.
@@ -320,6 +331,8 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   a.volMbar = (int)sp.volMbar;
   a.padShift = kPadShift;
   a.cachePolicy = opt.cachePolicy;
+  a.volume = pb.volume;
+  a.wideOffsets = (opt.wideOffsets || (uint64_t)pb.volume * (uint64_t)pb.elemSize > (1ull << 32)) ? 1 : 0;
   for (int i = 0; i < 2; i++) {
     cuttHipSplitRank& sr = a.split[i];
     sr.numSplit = 1;
@@ -352,14 +365,15 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   a.ldsElems = (int)slots;
   plan.ldsBytes = cuttHipPackedLdsBytes(&a);
   if (plan.ldsBytes > props.ldsPerBlock) return false;
-  choosePackedThreads(a.maxVol, props, opt.elemsPerThread, a.numThreads, a.elemsPerThread);
+  choosePackedThreads(a.maxVol, pb.elemSize, props, opt.elemsPerThread, a.numThreads, a.elemsPerThread);
   if (a.numThreads == 0) return false;
   // Work items per workgroup: amortise the table load without starving the chip of workgroups.
   const int64_t items = sp.volMbar * (int64_t)a.split[0].numSplit * a.split[1].numSplit;
   if (items > 0x7fffffffll) return false;
   const int64_t residentPerCU =
       std::max<int64_t>(1, std::min<int64_t>((int64_t)(props.ldsPerCU / plan.ldsBytes),
-                                             props.maxThreadsPerCU / a.numThreads));
+                                             packedThreadsPerCU(props, pb.elemSize, a.elemsPerThread, a.wideOffsets) /
+                                                 a.numThreads));
   // Enough workgroups for several waves of residents, but several items each where possible: the
   // table slice a workgroup loads is reused by all of its items.
   if (opt.packedRounds > 0) {
@@ -530,9 +544,10 @@ void addPacked(const Problem& pb, bool fromReduced, const cuttHipDeviceProps& pr
 // Staged-block sizes (in elements) worth trying when Mmk has to be cut: about an eighth, a
 // quarter and a half of what one workgroup's LDS holds beside its tables.
 std::vector<int64_t> stagedTargets(const Problem& pb, const cuttHipDeviceProps& props) {
-  // what one workgroup can stage: LDS, and kMaxElemsPerThread elements on each of its lanes
+  // what one workgroup can stage: LDS, and the most elements its lanes can hold
   const int64_t cap = std::min<int64_t>({(int64_t)props.ldsPerBlock * 31 / 32 / pb.elemSize,
-                                         (int64_t)kMaxElemsPerThread * props.maxThreadsPerBlock, kMaxLdsSlots * 31 / 32});
+                                         (int64_t)maxElemsPerThread(pb.elemSize) * props.maxThreadsPerBlock,
+                                         kMaxLdsSlots * 31 / 32});
   return {cap / 4, cap / 2, cap};
 }
 

@@ -126,12 +126,13 @@ struct PlannerOptions {
   int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
   int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3/4: strips of 8 tiles along Mm
-  int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4 or 8
+  int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
   int maxItemsPerBlock = 4;  // Packed/PackedSplit: work items one workgroup handles at most
   bool policyOnly = false;  // (measuring planner) this variant differs only in the cache policy
   int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores
   int mbarOrder = 1;        // order of the Mbar ranks: 0 = input order, 1 = output order
+  bool wideOffsets = false; // Packed/PackedSplit: 64-bit address arithmetic also below 4 GB (tests)
   bool xcdAware = true;     // give every XCD (private L2) a contiguous chunk of the workgroup sequence
 };
 

@@ -288,6 +288,7 @@ void usage() {
   std::printf("-memcpy [int]    : time plain copies of this many elements\n");
   std::printf("-samples [int]   : tensors per rank (bench 3, 5) or per shape (bench 7) instead of the full count\n");
   std::printf("-nomemcpy        : do not time a same-size hipMemcpy beside each tensor\n");
+  std::printf("-bufelems [int]  : elements per buffer (default 420M of 4 bytes or 370M of 8 bytes)\n");
 }
 
 }  // namespace
@@ -295,7 +296,7 @@ void usage() {
 int main(int argc, char* argv[]) {
   int gpuid = -1, benchID = 0;
   uint64_t seed = 1;
-  long long memcpyElems = 0;
+  long long memcpyElems = 0, bufElemsArg = 0;
   std::vector<int> dimArg, permArg;
   bool argOk = true;
   int i = 1;
@@ -329,6 +330,9 @@ int main(int argc, char* argv[]) {
     } else if (a == "-memcpy" && i + 1 < argc) {
       memcpyElems = std::atoll(argv[i + 1]);
       i += 2;
+    } else if (a == "-bufelems" && i + 1 < argc) {
+      bufElemsArg = std::atoll(argv[i + 1]);
+      i += 2;
     } else if (a == "-elemsize" && i + 1 < argc) {
       elemSize = (size_t)std::atoi(argv[i + 1]);
       i += 2;
@@ -353,6 +357,7 @@ int main(int argc, char* argv[]) {
 
   // the reference's buffer sizes: 420M 4-byte or 370M 8-byte elements
   dataElems = (elemSize == 4 ? 420 : 370) * kMillion;
+  if (bufElemsArg > 0) dataElems = bufElemsArg;
   HIP_CHECK(hipMalloc(&dataIn, (size_t)dataElems * elemSize));
   HIP_CHECK(hipMalloc(&dataOut, (size_t)dataElems * elemSize));
   checker = new TensorChecker();

@@ -105,7 +105,8 @@ def emulate(cands, idx, data):
     num_threads, vol_mbar, items_per_block, pad_shift, lds_elems, xcd_chunk, elems_per_thread = sc[:7]
     splits = [sc[7:12], sc[12:17]]  # numSplit, slabFloor, slabRem, strideIn, strideOut
     assert num_threads % 64 == 0 and 64 <= num_threads <= 1024
-    assert elems_per_thread in (1, 2, 4, 8)
+    # 16 elements per lane exist for 4-byte elements only
+    assert elems_per_thread in (1, 2, 4, 8) or (elems_per_thread == 16 and data.dtype.itemsize == 4)
     off_in, off_out = _mbar_offsets(mbar, vol_mbar)
     ns0, ns1 = splits[0][0], splits[1][0]
     total_items = vol_mbar * ns0 * ns1

@@ -107,6 +107,60 @@ def test_forced_methods_large(gpu):
         cutt.set_method_override(0)
 
 
+def test_wide_offset_kernels_and_sixteen_per_lane(gpu):
+    # The packed kernel has a 64-bit-offset variant for tensors of 4 GB and more; CUTT_WIDE_OFFSETS=1
+    # runs it on small tensors.  4-byte elements also have a 16-elements-per-lane variant.
+    import os
+    import cutt_amd as cutt
+    cases = [((5, 7, 11, 13, 17, 31), (4, 2, 0, 5, 1, 3)), ((200000, 2, 50), (2, 1, 0)),
+             ((33, 5, 42, 15, 23, 10), (4, 5, 0, 2, 1, 3)), ((129, 3, 257, 31), (2, 0, 3, 1))]
+    try:
+        for env in ({"CUTT_WIDE_OFFSETS": "1"}, {"CUTT_ELEMS_PER_THREAD": "16"},
+                    {"CUTT_WIDE_OFFSETS": "1", "CUTT_ELEMS_PER_THREAD": "16"}):
+            os.environ.update(env)
+            for method in (cutt.METHOD_PACKED, cutt.METHOD_PACKEDSPLIT):
+                cutt.set_method_override(method)
+                for dim, perm in cases:
+                    for es in (4, 8):
+                        say("%s forced %s dim=%s es=%d" % (env, cutt.METHOD_NAMES[method], dim, es))
+                        st = gpu.stream_handle()
+                        rc, h = cutt.cuttPlan(len(dim), list(dim), list(perm), es, st)
+                        if rc != cutt.CUTT_SUCCESS:
+                            continue  # the forced method has no feasible candidate for this tensor
+                        info = cutt.get_plan_info(h)
+                        cutt.cuttDestroy(h)
+                        if "CUTT_ELEMS_PER_THREAD" in env and es == 4:
+                            assert info.elemsPerThread == 16
+                        if es == 8:
+                            assert info.elemsPerThread <= 8
+                        gpu.check_case(list(dim), list(perm), es)
+            for k in env:
+                del os.environ[k]
+    finally:
+        cutt.set_method_override(0)
+        os.environ.pop("CUTT_WIDE_OFFSETS", None)
+        os.environ.pop("CUTT_ELEMS_PER_THREAD", None)
+
+
+def test_register_table_matches_loaded_kernels(gpu):
+    # the planner's occupancy estimate rests on a table of registers per lane; it must describe
+    # the code object that is actually loaded
+    import ctypes
+    import cutt_amd
+    lib = ctypes.CDLL(cutt_amd.lib_path())
+    for es in (4, 8):
+        for e in (1, 2, 4, 8, 16):
+            if e == 16 and es == 8:
+                continue
+            for wide in (0, 1):
+                table = lib.cuttHipPackedRegsPerLane(es, e, wide)
+                loaded = lib.cuttHipPackedRegsPerLaneLoaded(es, e, wide)
+                say("packed kernel es=%d E=%d wide=%d: table %d, loaded %d" % (es, e, wide, table, loaded))
+                assert loaded > 0
+                # same allocation granule of 8 registers = same occupancy
+                assert (table + 7) // 8 == (loaded + 7) // 8, (es, e, wide, table, loaded)
+
+
 def test_random_ranks_up_to_15(gpu):
     # reference test2, seeded: random shapes and permutations for ranks 2..15
     rng = np.random.default_rng(2024)

@@ -63,3 +63,19 @@ def test_cutt_bench_ttc_suite():
     assert r.returncode == 0, r.stdout[-2000:]
     assert "bench OK" in r.stdout
     assert r.stdout.count("number of elements") == 57
+
+
+@pytest.mark.gpu
+def test_tensor_above_4GB_uses_wide_offsets():
+    # 671 088 640 doubles = 5.4 GB per buffer: byte offsets no longer fit 32 bits
+    import os
+    env = dict(os.environ, CUTT_FORCE_METHOD="packedsplit")
+    exe = os.path.join(BIN, "cutt_bench")
+    r = subprocess.run([exe, "-bufelems", "671088640", "-dim", "1024", "640", "1024", "-permutation", "2", "1", "0",
+                        "-nomemcpy"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600, env=env)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout and "method PackedSplit" in r.stdout
+    r = subprocess.run([exe, "-bufelems", "671088640", "-dim", "1024", "640", "1024", "-permutation", "2", "1", "0",
+                        "-nomemcpy", "-measure"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout
