@@ -509,13 +509,14 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   }
   const size_t lds = packedLdsBytes(a);
 
-  static bool ldsOptIn = false;  // benign if two threads race: the calls are idempotent
-  if (!ldsOptIn) {
-    int dev = 0;
+  // Function attributes are kept per device; benign if two threads race: the calls are idempotent.
+  static bool ldsOptInDone[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (!tracked || !ldsOptInDone[dev]) {
     hipDeviceProp_t prop;
-    hipError_t e = hipGetDevice(&dev);
-    if (e == hipSuccess) e = hipGetDeviceProperties(&prop, dev);
-    if (e != hipSuccess) return (int)e;
+    if (hipError_t e = hipGetDeviceProperties(&prop, dev); e != hipSuccess) return (int)e;
     const size_t m = prop.sharedMemPerBlock;
     int r = 0;
 #define CUTT_ALLOW(T, E)                                                  \
@@ -530,7 +531,7 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
 #undef CUTT_ALLOW
     if (r != 0) return r;
-    ldsOptIn = true;
+    if (tracked) ldsOptInDone[dev] = true;
   }
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(a->numThreads);

@@ -329,7 +329,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0);
   } else {
-    factor = 1.127 + 0.093 * (rdAmp - 1.0) + 0.223 * (wrAmp - 1.0) + 0.017 * partial + (es == 4 ? 0.038 : 0.0) -
+    factor = 1.09 + 0.093 * (rdAmp - 1.0) + 0.223 * (wrAmp - 1.0) + 0.017 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.072 : 0.0);
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;

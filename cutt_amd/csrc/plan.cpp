@@ -247,10 +247,25 @@ void enumerateOffsets(const std::vector<RadixDim>& dims, int64_t count, std::vec
 // lines at the ends of their runs meet in the same L2).
 void fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, cuttHipMbar& mb) {
   std::memset(&mb, 0, sizeof(mb));
-  int n = 0;
+  // Order of the Mbar ranks (first = fastest over consecutive work items):
+  //   0 input order, 1 output order, 2 the first input rank outside Mmk, then output order.
+  // Workgroups that run side by side on one XCD then touch neighbouring memory, and the lines at
+  // the unaligned edges of their runs are shared in the L2: with 2 on the read side for the
+  // nearest neighbour and on the write side for the next ones.
+  std::vector<int> order;
+  if (mbarOrder == 2)
+    for (int r = 0; r < pb.rank; r++)
+      if (!inMmk[r]) {
+        order.push_back(r);
+        break;
+      }
   for (int i = 0; i < pb.rank; i++) {
-    const int r = mbarOrder == 1 ? pb.perm[i] : i;
-    if (inMmk[r]) continue;
+    const int r = mbarOrder == 0 ? i : pb.perm[i];
+    if (inMmk[r] || (!order.empty() && mbarOrder == 2 && r == order[0])) continue;
+    order.push_back(r);
+  }
+  int n = 0;
+  for (int r : order) {
     mb.d[n].extent = (uint32_t)pb.dim[r];
     mb.d[n].strideIn = (uint32_t)pb.strideIn[r];
     mb.d[n].strideOut = (uint32_t)pb.strideOut[r];

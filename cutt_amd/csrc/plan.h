@@ -131,7 +131,9 @@ struct PlannerOptions {
   int maxItemsPerBlock = 4;  // Packed/PackedSplit: work items one workgroup handles at most
   bool policyOnly = false;  // (measuring planner) this variant differs only in the cache policy
   int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores
-  int mbarOrder = 1;        // order of the Mbar ranks: 0 = input order, 1 = output order
+  bool orderOnly = false;   // (measuring planner) this variant differs only in the order of the Mbar ranks
+  int mbarOrder = 2;        // order of the Mbar ranks: 0 = input order, 1 = output order,
+                            // 2 = first input rank outside Mmk, then output order
   bool wideOffsets = false; // Packed/PackedSplit: 64-bit address arithmetic also below 4 GB (tests)
   bool xcdAware = true;     // give every XCD (private L2) a contiguous chunk of the workgroup sequence
 };
