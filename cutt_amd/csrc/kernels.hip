@@ -9,23 +9,25 @@
  *  - every kernel moves opaque 4- or 8-byte words (uint32_t / uint64_t), one
  *    word per lane per access, so a wavefront touches 256 or 512 contiguous
  *    bytes per instruction when the run is long enough;
- *  - the per-rank decomposition of a workgroup's Mbar position is wave-uniform
- *    and read from the kernel-argument segment (scalar loads), instead of
- *    one-table-entry-per-lane plus cross-lane shuffles;
+ *  - the per-rank decomposition of a workgroup's Mbar position is wave-uniform:
+ *    lane k owns rank k, divides by precomputed multiply-high constants and the
+ *    wavefront sums the contributions with DPP adds (mbar_decode.h);
  *  - Tiled stages a 64x64 tile in LDS padded to 65 columns (conflict-free for
  *    both 4- and 8-byte words); each lane keeps 16 loads in flight; edges are handled by
  *    clamping indices, not by branches, so the memory instructions stay back to back;
  *  - Packed/PackedSplit take their index remap from tables the planner precomputed in device
- *    memory (input offset, output offset and LDS gather slot per staged element); a workgroup
- *    loads its slice once and keeps it in registers while it loops over its work items, so the
- *    loop body is load, LDS write, LDS read, store; the LDS buffer is skewed by one slot per
- *    2^padShift to break power-of-two bank strides;
+ *    memory (one input offset per contiguous input run, one output offset per contiguous output
+ *    run, an LDS gather slot per staged element); a workgroup derives its lanes' offsets once and
+ *    keeps them in registers while it loops over its work items, so the loop body is load, LDS
+ *    write, LDS read, store; the LDS buffer is skewed by one slot per 2^padShift to break
+ *    power-of-two bank strides;
  *  - workgroups are short-lived and small (a tile, or a few Mbar positions),
  *    thousands are in flight: on this chip that streams faster than a
  *    persistent grid-stride loop.
  *
  * All offsets are 32-bit element offsets (the API limits a tensor to fewer
- * than 2^31 elements); they are widened only when added to the base pointer.
+ * than 2^31 elements); the packed kernel turns them into 32-bit byte offsets
+ * from a wave-uniform base when the tensor is below 4 GB.
  */
 #include <hip/hip_runtime.h>
 

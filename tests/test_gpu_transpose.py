@@ -235,3 +235,45 @@ def test_special_bit_patterns(gpu):
     gpu.check_case([33, 65], [1, 0], 4, data=data)
     data8 = (data.astype(np.uint64) << np.uint64(32)) | np.uint64(0x7FF00000)
     gpu.check_case([33, 65], [1, 0], 8, data=data8)
+
+
+def test_plans_from_several_threads(gpu):
+    # the handle table is shared; creating, executing and destroying plans from several host
+    # threads at once must neither mix handles up nor corrupt results
+    import threading
+    import torch
+    import cutt_amd as cutt
+    import oracle
+    shapes = [((31, 17, 45), (2, 0, 1), 8), ((64, 33, 20), (1, 2, 0), 4), ((5, 7, 11, 13), (3, 1, 0, 2), 8),
+              ((129, 257), (1, 0), 4), ((8, 9, 10, 11), (2, 3, 0, 1), 4), ((300, 40, 7), (2, 1, 0), 8)]
+    errors = []
+
+    def worker(k):
+        try:
+            dim, perm, es = shapes[k % len(shapes)]
+            vol = int(np.prod(dim))
+            data = gpu.seeded(vol, es, seed=100 + k)
+            want = oracle.transpose(list(dim), list(perm), data)
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                d_in = gpu.to_device(data)
+                d_out = torch.full_like(d_in, -1)
+            stream.synchronize()
+            for _ in range(20):
+                rc, h = cutt.cuttPlan(len(dim), list(dim), list(perm), es, stream.cuda_stream)
+                assert rc == cutt.CUTT_SUCCESS
+                assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+                stream.synchronize()
+                assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+                assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_INVALID_PLAN
+            got = gpu.to_host(d_out, es)
+            assert np.array_equal(got, want), "thread %d: wrong bytes" % k
+        except Exception as e:  # collected and re-raised in the main thread
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
