@@ -11,7 +11,7 @@ the same-size device-to-device hipMemcpy measured in the same run, and a CPU
 baseline (the oracle's multithreaded transpose on the host cores).
 
   python bench.py [--gpus 1] [--steps K] [--warmup W]
-  python bench.py --all        # C1..C4 (+ forced PackedSplit on C4) -> gpurun_out/bench_all.json
+  python bench.py --all        # C1..C4 (+ forced PackedSplit on C4) -> bench_all.json in the --out folder
   python bench.py --sweep N    # first N tensors of the C5 sweep, cuttPlan and cuttPlanMeasure
 """
 import argparse
@@ -169,7 +169,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="run C1..C4 with both planners")
     ap.add_argument("--sweep", type=int, default=0, help="run the first N tensors of the C5 sweep")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
-    ap.add_argument("--out", default=os.path.join(ROOT, "gpurun_out"))
+    ap.add_argument("--out", default=os.path.join(ROOT, "bench_out"), help="folder for the --all / --sweep result files")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py measures one GPU: a transpose plan is bound to a single device and this "
