@@ -148,10 +148,27 @@ int cachePolicyOf(const Plan& p) {
 // line, so they pay off only when a workgroup uses (nearly) whole lines of what it reads;
 // streaming stores only when no written line is left partly covered by a workgroup.
 // (Not applied when CUTT_CACHE_POLICY pins the policy.)
-void chooseCachePolicy(Plan& p) {
+void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
   if (std::getenv("CUTT_CACHE_POLICY")) return;
   if (p.method == kTrivial) return;
-  const double lines = (double)p.pb.volume * p.pb.elemSize / 128.0;
+  // The memory-side cache decides for small and medium tensors (measured on random tensors of
+  // 4M-200M elements): while input and output fit it together, ordinary accesses are best
+  // (non-temporal ones go past it: 65-72 % of memcpy instead of 80-89 %); up to about 3.5 times
+  // its size per buffer, streaming the reads and letting the cache merge the writes wins clearly
+  // (at one cache size per buffer 99 % against 81 %); beyond that it no longer matters.
+  const double bytes = (double)p.pb.volume * p.pb.elemSize;
+  const double cache = (double)props.infinityCacheBytes;
+  if (cache > 0 && 2.0 * bytes <= cache) {
+    setCachePolicy(p, 0);
+    return;
+  }
+  const double lines = bytes / 128.0;
+  if (cache > 0 && bytes <= 3.5 * cache) {
+    // ... unless the plan reads each line from several requests (more than ~1.7 lines requested
+    // per line of data): then the re-reads must find the line in the caches (0.85-0.97 x)
+    setCachePolicy(p, p.model.rdLines < 1.7 * lines ? 1 : 0);
+    return;
+  }
   const bool wholeReads = p.model.rdLines <= 1.15 * lines;
   const bool wholeWrites = p.model.wrPartialLines == 0.0;
   setCachePolicy(p, wholeReads ? (wholeWrites ? 3 : 1) : 0);
@@ -247,7 +264,7 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
   const int best = chooseHeuristic(plans);
   if (best < 0) return CUTT_INTERNAL_ERROR;
-  chooseCachePolicy(plans[best]);
+  chooseCachePolicy(plans[best], props);
   return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
 }
 
@@ -272,7 +289,7 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   if (plans.empty()) return CUTT_INTERNAL_ERROR;
   for (Plan& p : plans) {
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
-    chooseCachePolicy(p);
+    chooseCachePolicy(p, props);
   }
 
   size_t numBytes = sizeofType;

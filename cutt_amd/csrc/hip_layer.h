@@ -39,6 +39,7 @@ typedef struct cuttHipDeviceProps {
   int memBusWidthBits;
   int l2Bytes;
   int maxGridX;
+  size_t infinityCacheBytes; /* memory-side cache behind the L2s (256 MB on gfx942/gfx950), 0 if unknown */
   char arch[64];            /* e.g. "gfx950:sramecc+:xnack-" */
 } cuttHipDeviceProps;
 

@@ -69,6 +69,9 @@ extern "C" int cuttHipGetDeviceProps(int device, cuttHipDeviceProps* p) {
   p->l2Bytes = d.l2CacheSize;
   p->maxGridX = d.maxGridSize[0];
   std::strncpy(p->arch, d.gcnArchName, sizeof(p->arch) - 1);
+  // The runtime does not report the memory-side cache; MI300X and MI355X have 256 MB.
+  if (std::strncmp(p->arch, "gfx94", 5) == 0 || std::strncmp(p->arch, "gfx95", 5) == 0)
+    p->infinityCacheBytes = (size_t)256 << 20;
   return 0;
 }
 

@@ -58,6 +58,7 @@ cuttHipDeviceProps defaultMI355XProps() {
   p.memBusWidthBits = 8192;
   p.l2Bytes = 4 * 1024 * 1024;
   p.maxGridX = 2147483647;
+  p.infinityCacheBytes = (size_t)256 << 20;
   std::strncpy(p.arch, "gfx950", sizeof(p.arch) - 1);
   return p;
 }

@@ -289,6 +289,7 @@ void usage() {
   std::printf("-samples [int]   : tensors per rank (bench 3, 5) or per shape (bench 7) instead of the full count\n");
   std::printf("-nomemcpy        : do not time a same-size hipMemcpy beside each tensor\n");
   std::printf("-bufelems [int]  : elements per buffer (default 420M of 4 bytes or 370M of 8 bytes)\n");
+  std::printf("-elems [int]     : (average) tensor volume of bench 3 and 5 (default 200M elements)\n");
 }
 
 }  // namespace
@@ -296,7 +297,7 @@ void usage() {
 int main(int argc, char* argv[]) {
   int gpuid = -1, benchID = 0;
   uint64_t seed = 1;
-  long long memcpyElems = 0, bufElemsArg = 0;
+  long long memcpyElems = 0, bufElemsArg = 0, avgElems = 200 * kMillion;
   std::vector<int> dimArg, permArg;
   bool argOk = true;
   int i = 1;
@@ -330,6 +331,9 @@ int main(int argc, char* argv[]) {
     } else if (a == "-memcpy" && i + 1 < argc) {
       memcpyElems = std::atoll(argv[i + 1]);
       i += 2;
+    } else if (a == "-elems" && i + 1 < argc) {
+      avgElems = std::atoll(argv[i + 1]);
+      i += 2;
     } else if (a == "-bufelems" && i + 1 < argc) {
       bufElemsArg = std::atoll(argv[i + 1]);
       i += 2;
@@ -345,6 +349,7 @@ int main(int argc, char* argv[]) {
     }
   }
   if (elemSize != 4 && elemSize != 8) argOk = false;
+  if (avgElems < 64) argOk = false;
   if (dimArg.size() != permArg.size()) argOk = false;
   bool known = benchID == 3 || benchID / 100 == 5 || benchID == 6 || benchID == 7;
   if (dimArg.empty() && !known && memcpyElems <= 0) argOk = false;
@@ -392,10 +397,10 @@ int main(int argc, char* argv[]) {
     }
     withData = false;
   } else if (benchID == 3) {
-    ok = bench3(rng, 200 * kMillion);
+    ok = bench3(rng, avgElems);
     withData = false;
   } else if (benchID / 100 == 5) {
-    ok = bench5(rng, 200 * kMillion, benchID % 100);
+    ok = bench5(rng, avgElems, benchID % 100);
   } else if (benchID == 6) {
     ok = bench6();
   } else if (benchID == 7) {
