@@ -336,6 +336,11 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor += 0.25 * tableBytes / (2.0 * bytes);
   }
   double t = tCopy * factor;
+  // Granularity: with few workgroups per CU the chip fills unevenly and drains slowly.  Measured on
+  // tensors of 2M-32M elements the time grows like 1 + (CUs * lanes/1024) / workgroups; for the
+  // tens of thousands of workgroups of a large tensor the term vanishes.
+  if (plan.numBlocks > 0)
+    t *= 1.0 + (double)props.cuCount * ((double)plan.numThreads / 1024.0) / (double)plan.numBlocks;
   if (plan.method == kPacked || plan.method == kPackedSplit) {
     // A workgroup spends about 1.3 us per work item regardless of the item's size (load latency,
     // two barriers, store issue); with small items that, not bandwidth, sets the time:
