@@ -50,6 +50,7 @@ class PlanInfo(ctypes.Structure):
         ("usMeasured", ctypes.c_double),
         ("numCandidates", ctypes.c_int), ("planMs", ctypes.c_double),
         ("cachePolicy", ctypes.c_int), ("elemsPerThread", ctypes.c_int),
+        ("rdEdgeDist", ctypes.c_double), ("wrEdgeDist", ctypes.c_double),
     ]
 
     @property

@@ -130,6 +130,8 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.cachePolicy = p.method == kTiled ? p.tiled.cachePolicy
                                       : (p.method == kTiledCopy ? p.tcopy.cachePolicy : p.packed.cachePolicy);
   o.elemsPerThread = p.packed.elemsPerThread;
+  o.rdEdgeDist = p.model.rdEdgeDist;
+  o.wrEdgeDist = p.model.wrEdgeDist;
 }
 
 void setCachePolicy(Plan& p, int policy) {

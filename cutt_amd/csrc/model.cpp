@@ -302,6 +302,38 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   const double blocksPerCU = std::max(1.0, std::min({byLds, byThreads, 32.0}));
   r.blocksPerCU = blocksPerCU;
 
+  // Distance, in work items, to the item that accesses the next run in memory.
+  if (plan.method == kPacked || plan.method == kPackedSplit) {
+    const cuttHipPackedArgs& a = plan.packed;
+    const Split& sp = plan.split;
+    const Problem& pb = plan.pb;
+    const double ns0 = a.split[0].numSplit, ns1 = a.split[1].numSplit;
+    auto mbarDist = [&](int rank, bool input) -> double {
+      double d = ns0 * ns1;
+      for (int k = 0; k < a.mbar.n; k++) {
+        const bool hit = input ? a.mbar.d[k].strideIn == (uint32_t)pb.strideIn[rank]
+                               : a.mbar.d[k].strideOut == (uint32_t)pb.strideOut[rank];
+        if (hit && a.mbar.d[k].extent == (uint32_t)pb.dim[rank]) return d;
+        d *= a.mbar.d[k].extent;
+      }
+      return 0.0;
+    };
+    auto edge = [&](bool input) -> double {
+      for (int i = 0; i < pb.rank; i++) {
+        const int rk = input ? i : pb.perm[i];
+        if (!sp.inMmk[rk]) return mbarDist(rk, input);
+        const int slot = sp.method == kPackedSplit ? sp.splitSlot(rk) : -1;
+        if (slot >= 0) return slot == 0 ? 1.0 : ns0;
+      }
+      return 0.0;
+    };
+    r.rdEdgeDist = edge(true);
+    r.wrEdgeDist = edge(false);
+  } else if (plan.method == kTiled || plan.method == kTiledCopy) {
+    r.rdEdgeDist = 1.0;   // the next tile along Mm is the next workgroup of the strip
+    r.wrEdgeDist = (double)(plan.method == kTiled ? plan.tiled.superM : plan.tcopy.superM);
+  }
+
   // --- time estimate ---
   // The estimate is "time of a same-size device-to-device copy" times an overhead factor that is
   // linear in a few transaction ratios.  The coefficients are a least-squares fit to the measured
@@ -313,8 +345,10 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   //    of edge tiles, whose clamped lanes repeat accesses that hit the L1, costs about a quarter
   //    of a real access.
   //  - Packed / PackedSplit: extra lines on the write side cost about twice as much as on the read
-  //    side (partly written lines have to be merged in the L2), 4-byte elements a little more per
-  //    byte than 8-byte ones, and a block cut into slabs a little more than a whole one.
+  //    side (partly written lines have to be merged in the L2), and up to three times as much when
+  //    the workgroup that writes the rest of the line runs hundreds of work items later (the line
+  //    leaves the L2 half written); 4-byte elements cost a little more per byte than 8-byte ones,
+  //    and a block cut into slabs a little more than a whole one.
   const double peakBW = (double)props.memClockKHz * 1e3 * 4.0 * (props.memBusWidthBits / 8.0);
   const double tCopy = 2.0 * bytes / (0.64 * peakBW);  // sustained rate of a large D2D copy
   const double lineBytes = bytes / kLineBytes;
@@ -329,8 +363,12 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0);
   } else {
-    factor = 1.09 + 0.093 * (rdAmp - 1.0) + 0.223 * (wrAmp - 1.0) + 0.017 * partial + (es == 4 ? 0.038 : 0.0) -
-             (plan.method == kPacked ? 0.072 : 0.0);
+    // A line shared by two runs is assembled (written) or reused (read) in the L2 only if the other
+    // run's workgroup comes soon: "far" rises from 0 at 32 work items apart to 1 at 512.
+    auto far = [](double dist) { return dist <= 0.0 ? 0.0 : std::min(1.0, std::max(0.0, (std::log2(dist) - 5.0) / 4.0)); };
+    factor = 1.07 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
+             (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
+             0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);

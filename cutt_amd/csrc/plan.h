@@ -83,6 +83,9 @@ struct ModelResult {
   double rdSectors = 0, wrSectors = 0; // 32-byte sectors touched
   double ldsCycles = 0;                // LDS cycles incl. bank conflicts, whole tensor
   double blocksPerCU = 0;
+  // Work items between the two workgroups that touch the two sides of a run's end (the next run
+  // in memory): small = the shared line is still in the L2 when its other part is accessed.
+  double rdEdgeDist = 0, wrEdgeDist = 0;
   double usPredicted = 0;              // predicted time in microseconds (ranking key)
 };
 

@@ -51,6 +51,9 @@ typedef struct cuttPlanInfo {
   double planMs;
   int cachePolicy;      /* 0 default, 1 non-temporal loads, 3 non-temporal loads and stores */
   int elemsPerThread;   /* Packed/PackedSplit */
+  /* cost model: work items between the accesses to the two parts of a line shared by neighbouring
+   * runs, on the read and on the write side (0 = no such neighbour) */
+  double rdEdgeDist, wrEdgeDist;
 } cuttPlanInfo;
 
 /* Describe an existing plan. */
