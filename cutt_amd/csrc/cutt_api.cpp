@@ -176,6 +176,33 @@ void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
   setCachePolicy(p, wholeReads ? (wholeWrites ? 3 : 1) : 0);
 }
 
+PlannerOptions plannerOptions(int forceMethod);
+
+// The order in which consecutive work items walk the Mbar ranks decides whether the lines shared
+// by neighbouring runs meet in the L2 on the read side or on the write side.  For the few
+// candidates the model ranks best, also estimate the other orders and keep the cheapest.
+// (Not applied when CUTT_MBAR_ORDER pins the order.)
+void refineMbarOrder(std::vector<Plan>& plans, const cuttHipDeviceProps& props, int force) {
+  if (std::getenv("CUTT_MBAR_ORDER")) return;
+  const PlannerOptions base = plannerOptions(force);
+  std::vector<int> idx;
+  for (int i = 0; i < (int)plans.size(); i++)
+    if (plans[i].method != kTrivial) idx.push_back(i);
+  std::sort(idx.begin(), idx.end(),
+            [&](int a, int b) { return plans[a].model.usPredicted < plans[b].model.usPredicted; });
+  for (size_t k = 0; k < idx.size() && k < 3; k++) {
+    Plan& p = plans[idx[k]];
+    for (int order : {0, 1, 2}) {
+      if (order == base.mbarOrder) continue;
+      PlannerOptions opt = base;
+      opt.mbarOrder = order;
+      Plan q;
+      if (!rebuildPlan(p, props, opt, q) || !estimatePlan(q, props, 10)) continue;
+      if (q.model.usPredicted < p.model.usPredicted) p = std::move(q);
+    }
+  }
+}
+
 // Index of the candidate with the smallest predicted time; Trivial always wins and ties go to
 // the later candidate (reference src/cuttplan.cpp:700-768).
 int chooseHeuristic(const std::vector<Plan>& plans) {
@@ -264,6 +291,7 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
   for (Plan& p : plans)
     if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
+  refineMbarOrder(plans, props, force);
   const int best = chooseHeuristic(plans);
   if (best < 0) return CUTT_INTERNAL_ERROR;
   chooseCachePolicy(plans[best], props);

@@ -330,8 +330,32 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     r.rdEdgeDist = edge(true);
     r.wrEdgeDist = edge(false);
   } else if (plan.method == kTiled || plan.method == kTiledCopy) {
-    r.rdEdgeDist = 1.0;   // the next tile along Mm is the next workgroup of the strip
-    r.wrEdgeDist = (double)(plan.method == kTiled ? plan.tiled.superM : plan.tcopy.superM);
+    // Distances in workgroups (one tile each).  Along a tiled rank the next run belongs to the next
+    // tile: the next workgroup along Mm, superM workgroups on along Mk (strip order).  A rank that
+    // fits one tile ends its runs at the rank's end: the next run belongs to another Mbar position.
+    const bool copy = plan.method == kTiledCopy;
+    const cuttHipMbar& mb = copy ? plan.tcopy.mbar : plan.tiled.mbar;
+    const double tilesM = copy ? plan.tcopy.tilesM : plan.tiled.tilesM;
+    const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
+    const double superM = copy ? plan.tcopy.superM : plan.tiled.superM;
+    const Problem& pb = plan.pb;
+    auto mbarDist = [&](int rank, bool input) -> double {
+      double d = tilesM * tilesK;
+      for (int k = 0; k < mb.n; k++) {
+        const bool hit = input ? mb.d[k].strideIn == (uint32_t)pb.strideIn[rank]
+                               : mb.d[k].strideOut == (uint32_t)pb.strideOut[rank];
+        if (hit && mb.d[k].extent == (uint32_t)pb.dim[rank]) return d;
+        d *= mb.d[k].extent;
+      }
+      return 0.0;
+    };
+    // input runs lie along rank 0; output runs along the first output rank (Tiled) or rank 0 (TiledCopy)
+    r.rdEdgeDist = tilesM > 1 ? 1.0 : (pb.rank > 1 ? mbarDist(1, true) : 0.0);
+    if (copy) {
+      r.wrEdgeDist = tilesM > 1 ? 1.0 : (pb.rank > 1 ? mbarDist(pb.perm[1], false) : 0.0);
+    } else {
+      r.wrEdgeDist = tilesK > 1 ? std::min(superM, tilesM) : (pb.rank > 1 ? mbarDist(pb.perm[1], false) : 0.0);
+    }
   }
 
   // --- time estimate ---
@@ -354,6 +378,16 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
   const double lineBytes = bytes / kLineBytes;
   const double rdAmp = r.rdLines / lineBytes, wrAmp = r.wrLines / lineBytes;
   const double partial = r.wrPartialLines / lineBytes;
+  // A line shared by two runs is assembled (written) or reused (read) in the L2 only if the other
+  // run's workgroup comes soon: "far" rises from 0 when the workgroups in between move one L2's
+  // worth of data (4 MB per XCD) to 1 at sixteen times that.
+  const double itemBytes = (plan.method == kTiled || plan.method == kTiledCopy)
+                               ? 2.0 * kTile * kTile * es
+                               : 2.0 * (double)plan.packed.maxVol * es;
+  const double l2Bytes = props.l2Bytes > 0 ? (double)props.l2Bytes : 4.0 * 1024 * 1024;
+  auto far = [&](double dist) {
+    return dist <= 0.0 ? 0.0 : std::min(1.0, std::max(0.0, std::log2(dist * itemBytes / l2Bytes) / 4.0));
+  };
   double factor;
   if (plan.method == kTiled || plan.method == kTiledCopy) {
     const bool copy = plan.method == kTiledCopy;
@@ -361,11 +395,8 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
     const double waste = tilesM * tilesK * (double)plan.split.volMbar * kTile * kTile / (double)plan.pb.volume - 1.0;
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
-             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0);
+             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
   } else {
-    // A line shared by two runs is assembled (written) or reused (read) in the L2 only if the other
-    // run's workgroup comes soon: "far" rises from 0 at 32 work items apart to 1 at 512.
-    auto far = [](double dist) { return dist <= 0.0 ? 0.0 : std::min(1.0, std::max(0.0, (std::log2(dist) - 5.0) / 4.0)); };
     factor = 1.07 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
