@@ -400,6 +400,9 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor = 1.07 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
+    // Sixteen elements per lane leave room for one workgroup per CU only; measured about 8 % slower
+    // than the counters alone predict.
+    if (plan.packed.elemsPerThread > 8) factor += 0.08;
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);
