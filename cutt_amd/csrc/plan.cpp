@@ -39,11 +39,6 @@ const char* methodName(int method) {
   }
 }
 
-uint32_t divMagic(uint32_t d) {
-  if (d < 2) return 0;
-  return (uint32_t)(((1ull << 32) + d - 1) / d);
-}
-
 cuttHipDeviceProps defaultMI355XProps() {
   cuttHipDeviceProps p;
   std::memset(&p, 0, sizeof(p));

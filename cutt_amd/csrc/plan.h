@@ -153,9 +153,6 @@ bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const Planner
 // Default device description of one MI355X, used when no GPU is present (tests, offline planning).
 cuttHipDeviceProps defaultMI355XProps();
 
-// magic = ceil(2^32 / d) for the multiply-high division used by the packed kernel (d >= 2).
-uint32_t divMagic(uint32_t d);
-
 }  // namespace cutt
 
 #endif  // CUTT_PLAN_H
