@@ -277,3 +277,36 @@ def test_plans_from_several_threads(gpu):
     for t in threads:
         t.join()
     assert not errors, errors
+
+
+def test_execute_under_graph_capture(gpu):
+    # cuttExecute only launches a kernel (or a device-to-device copy) on the plan's stream, so it
+    # can be captured into a HIP graph; every replay must transpose what the input holds then
+    import torch
+    import cutt_amd as cutt
+    import oracle
+    for dim, perm, es in (((129, 3, 257, 31), (2, 0, 3, 1), 8), ((64, 96, 50), (1, 2, 0), 4), ((40, 50, 60), (0, 1, 2), 8)):
+        vol = int(np.prod(dim))
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            d_in = gpu.to_device(gpu.seeded(vol, es, seed=1))
+            d_out = torch.full_like(d_in, -1)
+            rc, h = cutt.cuttPlan(len(dim), list(dim), list(perm), es, stream.cuda_stream)
+            assert rc == cutt.CUTT_SUCCESS
+            # first launch outside the capture: it sets kernel attributes once per process and device
+            assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+        for seed in (2, 3, 4):
+            data = gpu.seeded(vol, es, seed=seed)
+            d_in.copy_(gpu.to_device(data))
+            d_out.fill_(-1)
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            say("graph replay dim=%s es=%d seed=%d" % (dim, es, seed))
+            assert np.array_equal(gpu.to_host(d_out, es), oracle.transpose(list(dim), list(perm), data))
+        del graph
+        assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
