@@ -217,6 +217,8 @@ const char* cuttHipErrorString(int err);
 int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);
+/* One-time kernel attribute setup of the packed kernels on the current device (idempotent). */
+int cuttHipPreparePacked(void);
 
 #ifdef __cplusplus
 }

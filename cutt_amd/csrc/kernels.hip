@@ -470,6 +470,37 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   return (int)hipGetLastError();
 }
 
+// Lets the packed kernels use more than the default 64 KB of dynamic LDS on the current device.
+// Called when a packed plan is activated (so that a plan's first cuttExecute already is a plain
+// kernel launch) and, as a cheap check, before every launch.
+extern "C" int cuttHipPreparePacked(void) {
+  // Function attributes are kept per device; benign if two threads race: the calls are idempotent.
+  static bool ldsOptInDone[64] = {};
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  const bool tracked = dev >= 0 && dev < 64;
+  if (!tracked || !ldsOptInDone[dev]) {
+    hipDeviceProp_t prop;
+    if (hipError_t e = hipGetDeviceProperties(&prop, dev); e != hipSuccess) return (int)e;
+    const size_t m = prop.sharedMemPerBlock;
+    int r = 0;
+#define CUTT_ALLOW(T, E)                                                  \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, false>, m);         \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, true>, m);          \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, true>, m);          \
+  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, true>, m)
+    CUTT_ALLOW(uint32_t, 1); CUTT_ALLOW(uint32_t, 2); CUTT_ALLOW(uint32_t, 4); CUTT_ALLOW(uint32_t, 8);
+    CUTT_ALLOW(uint32_t, 16);
+    CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
+#undef CUTT_ALLOW
+    if (r != 0) return r;
+    if (tracked) ldsOptInDone[dev] = true;
+  }
+  return 0;
+}
+
 extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, void* out, void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
@@ -511,30 +542,7 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
   }
   const size_t lds = packedLdsBytes(a);
 
-  // Function attributes are kept per device; benign if two threads race: the calls are idempotent.
-  static bool ldsOptInDone[64] = {};
-  int dev = 0;
-  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
-  const bool tracked = dev >= 0 && dev < 64;
-  if (!tracked || !ldsOptInDone[dev]) {
-    hipDeviceProp_t prop;
-    if (hipError_t e = hipGetDeviceProperties(&prop, dev); e != hipSuccess) return (int)e;
-    const size_t m = prop.sharedMemPerBlock;
-    int r = 0;
-#define CUTT_ALLOW(T, E)                                                  \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, false>, m);         \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, false>, m);         \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, false>, m);         \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 0, true>, m);          \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 1, true>, m);          \
-  if (r == 0) r = allowLargeLds(packedKernel<T, E, 3, true>, m)
-    CUTT_ALLOW(uint32_t, 1); CUTT_ALLOW(uint32_t, 2); CUTT_ALLOW(uint32_t, 4); CUTT_ALLOW(uint32_t, 8);
-    CUTT_ALLOW(uint32_t, 16);
-    CUTT_ALLOW(uint64_t, 1); CUTT_ALLOW(uint64_t, 2); CUTT_ALLOW(uint64_t, 4); CUTT_ALLOW(uint64_t, 8);
-#undef CUTT_ALLOW
-    if (r != 0) return r;
-    if (tracked) ldsOptInDone[dev] = true;
-  }
+  if (int r = cuttHipPreparePacked(); r != 0) return r;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(a->numThreads);
   const bool wide = a->wideOffsets != 0;

@@ -780,6 +780,7 @@ int Plan::activate() {
   if (method != kPacked && method != kPackedSplit) return 0;
   if (dTables) return 0;
   if (!buildTables()) return -1;
+  if (int e = cuttHipPreparePacked(); e != 0) return e;
   // One allocation: [rowIn | rowOut | shIdx] per class, each piece 16-byte aligned.
   auto align16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
   size_t total = 0;

@@ -293,7 +293,7 @@ def test_execute_under_graph_capture(gpu):
             d_out = torch.full_like(d_in, -1)
             rc, h = cutt.cuttPlan(len(dim), list(dim), list(perm), es, stream.cuda_stream)
             assert rc == cutt.CUTT_SUCCESS
-            # first launch outside the capture: it sets kernel attributes once per process and device
+            # first launch outside the capture: the runtime loads the library's code object then
             assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
