@@ -390,9 +390,9 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
       v.tiledOrder = 2;                                  // tiles along the output run fastest
       variants.push_back(v);
     } else {
-      for (int ipb : {1, 2, 8}) {
+      for (int ipb : {1, 2, 4, 8}) {
         PlannerOptions v = base;
-        if (ipb == v.maxItemsPerBlock) continue;
+        if (ipb == plans[best].packed.itemsPerBlock) continue;
         v.maxItemsPerBlock = ipb;
         variants.push_back(v);
       }

@@ -56,6 +56,8 @@ __device__ __forceinline__ void stg(T* p, T v) {
 constexpr int kTile = 64;             // tile edge in elements
 constexpr int kTileThreads = 256;     // 4 wavefronts
 constexpr int kTileRows = kTile * kTile / kTileThreads;  // rows per lane: 16
+constexpr int kGroupRows = 4;                            // rows per lane in one skippable group
+constexpr int kRowGroups = kTileRows / kGroupRows;       // 4 groups of 16 tile rows each
 constexpr int kWaves = kTileThreads / 64;
 
 // Workgroup index -> (tile along Mm, tile along Mk, Mbar position).  Returns false for the
@@ -139,20 +141,36 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
   const uint32_t wM = min((uint32_t)kTile, volMm - m0) - 1;  // last valid column / row inside the tile
   const uint32_t wK = min((uint32_t)kTile, volMk - k0) - 1;
 
+  // The 16 rows of a lane come in kRowGroups groups of 4; group g covers tile rows 16g..16g+15
+  // over the four waves.  An edge tile skips the groups that lie entirely beyond its valid part
+  // (a test that is uniform over the workgroup), so that a thin edge costs a quarter of a tile's
+  // instructions, not all of them; inside a group the clamping above still applies.
+  const uint32_t groupsK = (wK >> 4) + 1, groupsM = (wM >> 4) + 1;
+
   // Read: lanes run along input rank 0, rows along the Mk rank.
   {
     const uint32_t cx = min(lane, wM);
     const T* src = in + (offIn + m0 + cx);
     T v[kTileRows];
 #pragma unroll
-    for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = min(wave + kWaves * j, wK);
-      v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
+    for (int g = 0; g < kRowGroups; g++) {
+      if ((uint32_t)g < groupsK) {
+#pragma unroll
+        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+          const uint32_t r = min(wave + kWaves * j, wK);
+          v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
+        }
+      }
     }
 #pragma unroll
-    for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = min(wave + kWaves * j, wK);
-      tile[r][cx] = v[j];
+    for (int g = 0; g < kRowGroups; g++) {
+      if ((uint32_t)g < groupsK) {
+#pragma unroll
+        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+          const uint32_t r = min(wave + kWaves * j, wK);
+          tile[r][cx] = v[j];
+        }
+      }
     }
   }
   __syncthreads();
@@ -162,14 +180,24 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
     T* dst = out + (offOut + k0 + ck);
     T v[kTileRows];
 #pragma unroll
-    for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = min(wave + kWaves * j, wM);
-      v[j] = tile[ck][r];
+    for (int g = 0; g < kRowGroups; g++) {
+      if ((uint32_t)g < groupsM) {
+#pragma unroll
+        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+          const uint32_t r = min(wave + kWaves * j, wM);
+          v[j] = tile[ck][r];
+        }
+      }
     }
 #pragma unroll
-    for (int j = 0; j < kTileRows; j++) {
-      const uint32_t r = min(wave + kWaves * j, wM);
-      stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
+    for (int g = 0; g < kRowGroups; g++) {
+      if ((uint32_t)g < groupsM) {
+#pragma unroll
+        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+          const uint32_t r = min(wave + kWaves * j, wM);
+          stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
+        }
+      }
     }
   }
 }
@@ -195,16 +223,28 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
   const T* src = in + (offIn + m0 + cx);
   T* dst = out + (offOut + m0 + cx);
 
+  // Row groups that lie beyond the tile's valid rows are skipped, as in the tiled kernel.
+  const uint32_t groupsK = (wK >> 4) + 1;
   T v[kTileRows];
 #pragma unroll
-  for (int j = 0; j < kTileRows; j++) {
-    const uint32_t r = min(wave + kWaves * j, wK);
-    v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
+  for (int g = 0; g < kRowGroups; g++) {
+    if ((uint32_t)g < groupsK) {
+#pragma unroll
+      for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+        const uint32_t r = min(wave + kWaves * j, wK);
+        v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
+      }
+    }
   }
 #pragma unroll
-  for (int j = 0; j < kTileRows; j++) {
-    const uint32_t r = min(wave + kWaves * j, wK);
-    stg<NT>(dst + (k0 + r) * a.strideOutK, v[j]);
+  for (int g = 0; g < kRowGroups; g++) {
+    if ((uint32_t)g < groupsK) {
+#pragma unroll
+      for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
+        const uint32_t r = min(wave + kWaves * j, wK);
+        stg<NT>(dst + (k0 + r) * a.strideOutK, v[j]);
+      }
+    }
   }
 }
 

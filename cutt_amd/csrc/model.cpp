@@ -393,7 +393,15 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const bool copy = plan.method == kTiledCopy;
     const double tilesM = copy ? plan.tcopy.tilesM : plan.tiled.tilesM;
     const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
-    const double waste = tilesM * tilesK * (double)plan.split.volMbar * kTile * kTile / (double)plan.pb.volume - 1.0;
+    // Issued lane-slots over useful ones: a request is 64 lanes wide whatever the tile's width, and
+    // an edge tile issues its rows in groups of 16 (loads run over Mk rows; the stores of a Tiled
+    // plan run over Mm rows, those of a TiledCopy plan over Mk rows again).
+    const double volMm = copy ? plan.tcopy.volMm : plan.tiled.volMm;
+    const double volMk = copy ? plan.tcopy.volMk : plan.tiled.volMk;
+    auto rows16 = [](double n) { return std::ceil(n / 16.0) * 16.0; };
+    const double rdSlots = tilesM * kTile * rows16(volMk);
+    const double wrSlots = copy ? rdSlots : rows16(volMm) * tilesK * kTile;
+    const double waste = 0.5 * (rdSlots + wrSlots) / (volMm * volMk) - 1.0;
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
   } else {
