@@ -25,9 +25,10 @@
  *    thousands are in flight: on this chip that streams faster than a
  *    persistent grid-stride loop.
  *
- * All offsets are 32-bit element offsets (the API limits a tensor to fewer
- * than 2^31 elements); the packed kernel turns them into 32-bit byte offsets
- * from a wave-uniform base when the tensor is below 4 GB.
+ * All offsets are unsigned 32-bit element offsets (the API limits a tensor to
+ * fewer than 2^32 elements; every true offset is below the volume, so the
+ * modular sums are exact); the packed kernel turns them into 32-bit byte
+ * offsets from a wave-uniform base when the tensor is below 4 GB.
  */
 #include <hip/hip_runtime.h>
 
@@ -549,7 +550,7 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
        a->elemsPerThread != 8 && !(a->elemsPerThread == 16 && a->elemSize == 4)) ||
       (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) ||
       a->padShift > 31 || a->ldsElems < 1 || a->ldsElems > 65536 || !mbarOk(a->mbar) || a->volume < 1 ||
-      a->volume > 0x7fffffffll ||
+      a->volume > 0xffffffffll ||
       // 32-bit byte offsets reach 4 GB
       (!a->wideOffsets && (uint64_t)a->volume * (uint64_t)a->elemSize > (1ull << 32)))
     return (int)hipErrorInvalidValue;

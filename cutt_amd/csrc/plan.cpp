@@ -86,7 +86,8 @@ void reduceRanks(int rank, const int* dim, const int* perm, std::vector<int>& re
   // Groups of output ranks whose input ranks are consecutive and increasing.
   std::vector<int> first, vol;
   for (int j = 0; j < rank; j++) {
-    if (j > 0 && perm[j] == perm[j - 1] + 1) {
+    // (a fused extent must still fit an int; beyond that the ranks stay apart)
+    if (j > 0 && perm[j] == perm[j - 1] + 1 && (int64_t)vol.back() * dim[perm[j]] < (1ll << 31)) {
       vol.back() *= dim[perm[j]];
     } else {
       first.push_back(perm[j]);
@@ -241,7 +242,7 @@ void enumerateOffsets(const std::vector<RadixDim>& dims, int64_t count, std::vec
 // remaining index space: mbarOrder 0 = input order (consecutive workgroups read neighbouring
 // memory), 1 = output order (they write neighbouring memory, so the partly written 128-byte
 // lines at the ends of their runs meet in the same L2).
-void fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, cuttHipMbar& mb) {
+bool fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, cuttHipMbar& mb) {
   std::memset(&mb, 0, sizeof(mb));
   // Order of the Mbar ranks (first = fastest over consecutive work items):
   //   0 input order, 1 output order, 2 the first input rank outside Mmk, then output order.
@@ -268,7 +269,9 @@ void fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, 
     n++;
   }
   mb.n = n;
-  cuttHipFinishMbar(&mb);  // cannot fail: the extents multiply to at most the tensor's volume < 2^31
+  // Fails only when the extents multiply to 2^31 or more (a tensor of 2^31 elements and more with
+  // a tiny Mmk); such a candidate is dropped.
+  return cuttHipFinishMbar(&mb) == 0;
 }
 
 // Extent of rank r inside one staged block whose split ranks have the slab sizes slab[0..1].
@@ -406,8 +409,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
     plan.numBlocks = (int64_t)a.xcdChunk * kNumXcd;
   }
   plan.numThreads = a.numThreads;
-  fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
-  return true;
+  return fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
 }
 
 // Ordering of a tiled launch: fills order, super-tile shape and the per-XCD chunk; returns the
@@ -461,7 +463,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
-    fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
+    if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
     plan.ldsBytes = (size_t)kTile * (kTile + 1) * pb.elemSize;
   } else {
     cuttHipTiledCopyArgs& a = plan.tcopy;
@@ -479,7 +481,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
-    fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
+    if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
     plan.ldsBytes = 0;
   }
   plan.numThreads = 256;
@@ -710,8 +712,11 @@ bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const Planner
 
 bool createPlans(const Problem& orig, const Problem& red, const cuttHipDeviceProps& props,
                  const PlannerOptions& opt, std::vector<Plan>& plans) {
-  if (red.rank == 1) {
-    // Everything fused into one rank: a plain copy is the only candidate.
+  bool identity = true;
+  for (int i = 0; i < red.rank; i++) identity = identity && red.perm[i] == i;
+  if (identity) {
+    // Everything fuses into one rank (or would, if the fused extent still fitted an int): a plain
+    // copy is the only candidate.
     addTrivial(red, plans);
     return true;
   }

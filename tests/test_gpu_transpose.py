@@ -310,3 +310,21 @@ def test_execute_under_graph_capture(gpu):
             assert np.array_equal(gpu.to_host(d_out, es), oracle.transpose(list(dim), list(perm), data))
         del graph
         assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+
+
+def test_identity_of_2_to_31_elements_is_a_copy(gpu):
+    # the fused extent no longer fits an int, so the ranks stay apart; the plan is still Trivial
+    import torch
+    import cutt_amd as cutt
+    st = gpu.stream_handle()
+    n = 65536 * 32768
+    a = torch.empty(n, dtype=torch.int32, device="cuda")
+    a.random_()
+    b = torch.zeros_like(a)
+    rc, h = cutt.cuttPlan(2, (65536, 32768), (0, 1), 4, st)
+    assert rc == cutt.CUTT_SUCCESS
+    assert cutt.get_plan_info(h).method_name == "Trivial"
+    assert cutt.cuttExecute(h, a.data_ptr(), b.data_ptr()) == cutt.CUTT_SUCCESS
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS

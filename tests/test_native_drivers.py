@@ -79,3 +79,27 @@ def test_tensor_above_4GB_uses_wide_offsets():
                         "-nomemcpy", "-measure"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
     assert r.returncode == 0, r.stdout[-2000:]
     assert "bench OK" in r.stdout
+
+
+@pytest.mark.gpu
+def test_tensor_of_2_to_31_elements_and_more():
+    # 2 148 353 100 four-byte elements (8.6 GB per buffer) and 2 147 581 963 eight-byte ones
+    # (17.2 GB per buffer): more than the reference's int volumes hold; checked on the device by
+    # closed form like every other tensor of the driver.
+    import os
+    exe = os.path.join(BIN, "cutt_bench")
+    big4 = ["-elemsize", "4", "-bufelems", "2148353100", "-dim", "1291", "1290", "1290", "-permutation", "2", "0", "1",
+            "-nomemcpy"]
+    for force, extra, want in ((None, [], "method "), ("tiled", [], "method Tiled"),
+                               ("packedsplit", [], "method PackedSplit"), (None, ["-measure"], "method ")):
+        env = dict(os.environ)
+        if force:
+            env["CUTT_FORCE_METHOD"] = force
+        r = subprocess.run([exe] + big4 + extra, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True,
+                           timeout=600, env=env)
+        assert r.returncode == 0, r.stdout[-2000:]
+        assert "bench OK" in r.stdout and want in r.stdout
+    r = subprocess.run([exe, "-bufelems", "2147581963", "-dim", "46341", "46343", "-permutation", "1", "0", "-nomemcpy"],
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout

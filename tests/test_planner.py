@@ -103,6 +103,24 @@ def test_identity_gives_trivial(cutt):
             assert len(c) == 1 and c.info(0).method_name == "Trivial"
 
 
+def test_two_to_the_31_elements_and_more(cutt):
+    # Beyond the reference's int volumes: up to 2^32 - 1 elements are planned.  A fused extent must
+    # still fit an int, so the ranks of such an identity stay apart and it is still a plain copy.
+    assert cutt.reduce_ranks((46341, 46341), (0, 1)) == ([46341, 46341], [0, 1])
+    assert cutt.reduce_ranks((4, 46341, 46341), (1, 2, 0)) == ([4, 46341, 46341], [1, 2, 0])
+    with cutt.Candidates((65536, 32768), (0, 1), 4) as c:
+        assert len(c) == 1 and c.info(0).method_name == "Trivial"
+    infos, best = method_set(cutt, (1291, 1290, 1290), (2, 0, 1), 4)
+    names = {i.method_name for i in infos}
+    assert "Tiled" in names and "PackedSplit" in names
+    for i in infos:
+        assert 0 < i.volMbar < 2 ** 31 and i.numBlocks < 2 ** 31
+    # every Mbar position must stay below 2^31 for the kernels' division: a candidate whose
+    # staged block is tiny is dropped, the others remain
+    infos, best = method_set(cutt, (2, 2, 32768, 32767), (1, 0, 3, 2), 8)
+    assert infos and all(i.volMbar < 2 ** 31 for i in infos)
+
+
 def test_invalid_problems_rejected(cutt):
     for dim, perm, es in [((4, 4), (0, 0), 4), ((4, 1), (1, 0), 4), ((4, 4), (1, 0), 2), ((4,), (0,), 4),
                           ((4, 4), (1, 2), 8), ((65536, 65536), (1, 0), 4)]:
