@@ -411,6 +411,9 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // Sixteen elements per lane leave room for one workgroup per CU only; measured about 8 % slower
     // than the counters alone predict.
     if (plan.packed.elemsPerThread > 8) factor += 0.08;
+    // Large items run faster than their counters say (fewer barriers and table loads per byte):
+    // measured 5-8 % between 4 KB and 64 KB of staged data.
+    factor -= 0.06 * (double)plan.ldsBytes / 65536.0;
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);
