@@ -254,7 +254,8 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
 // ---------------------------------------------------------------------------
 
 // E = elements per lane.  Every lane keeps its E table entries in registers, so that the loop
-// over work items does no index arithmetic beyond adding the item's base offsets.
+// over work items does no index arithmetic beyond adding the item's base offsets; the loop is
+// software-pipelined (an item's loads are in flight while the previous one is gathered and stored).
 // WIDE = false: the tensor is smaller than 4 GB, so the lanes keep 32-bit byte offsets and every
 // access is "uniform 64-bit base + 32-bit lane offset" (no per-access 64-bit address registers).  WIDE = true:
 // element offsets and 64-bit address arithmetic.
@@ -282,51 +283,59 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // out back to back.
   uint32_t inOff[E], outOff[E];  // global offsets: bytes (narrow) or elements (wide)
   uint32_t shSlot[E];            // byte offset of the LDS slot an output element is taken from
-  uint32_t last = 0;             // last element index of the loaded class
-  int loaded = -1;
+  uint32_t last = 0;             // last element index of the class whose data is being loaded
   const MbarLane mbarLane = loadMbarLane(a.mbar, tid & 63);
   const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
-  for (uint32_t w = w0; w < w1; w++) {
+
+  // Work item w -> slab class and the item's base offsets (all wave-uniform).
+  auto locate = [&](uint32_t w, int& c, uint32_t& offIn, uint32_t& offOut) __attribute__((always_inline)) {
     const uint32_t t = fastDivide(w, div0.mul, div0.shift, div0.add);
     const uint32_t s0 = w - t * ns0;
     const uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
     const uint32_t s1 = t - m * ns1;
-    const int c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
+    c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
     const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
     const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
-
-    uint32_t offIn, offOut;
     mbarOffsets(mbarLane, m, offIn, offOut);
     offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
     offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
-
-    if (c != loaded) {  // wave-uniform: the class changes at most a few times per workgroup
-      const cuttHipPackedClass& k = a.cls[c];
-      last = (uint32_t)k.vol - 1;
-      const uint32_t inCont = (uint32_t)k.inCont, outCont = (uint32_t)k.outCont;
-      const uint32_t* gIn = k.rowIn;
-      const uint32_t* gOut = k.rowOut;
-      const uint16_t* gSh = k.shIdx;
+  };
+  // The lane's table entries of class c: the read side (input offsets, element count) and the
+  // write side (output offsets, LDS gather slots) are fetched separately, because the next item's
+  // loads go out while the current item's stores are still to come.
+  auto loadReadSide = [&](int c) __attribute__((always_inline)) {
+    const cuttHipPackedClass& k = a.cls[c];
+    last = (uint32_t)k.vol - 1;
+    const uint32_t inCont = (uint32_t)k.inCont;
+    const uint32_t* gIn = k.rowIn;
 #pragma unroll
-      for (int j = 0; j < E; j++) {
-        const uint32_t p = min(tid + j * nt, last);
-        const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
-        const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
-        // uniform base + 32-bit lane offset here too (the tables are far smaller than 4 GB)
-        const uint32_t rowI = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gIn) + ri * 4u);
-        const uint32_t rowO = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gOut) + ro * 4u);
-        const uint32_t sh = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const unsigned char*>(gSh) + p * 2u);
-        inOff[j] = (rowI + (p - ri * inCont)) * kScale;
-        outOff[j] = (rowO + (p - ro * outCont)) * kScale;
-        shSlot[j] = sh * (uint32_t)sizeof(T);
-      }
-      loaded = c;
+    for (int j = 0; j < E; j++) {
+      const uint32_t p = min(tid + j * nt, last);
+      const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
+      // uniform base + 32-bit lane offset here too (the tables are far smaller than 4 GB)
+      const uint32_t rowI = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gIn) + ri * 4u);
+      inOff[j] = (rowI + (p - ri * inCont)) * kScale;
     }
-    // wave-uniform bases of this item
-    const unsigned char* srcB = reinterpret_cast<const unsigned char*>(in + offIn);
-    unsigned char* dstB = reinterpret_cast<unsigned char*>(out + offOut);
-
-    T v[E];
+  };
+  auto loadWriteSide = [&](int c) __attribute__((always_inline)) {
+    const cuttHipPackedClass& k = a.cls[c];
+    const uint32_t lastP = (uint32_t)k.vol - 1;
+    const uint32_t outCont = (uint32_t)k.outCont;
+    const uint32_t* gOut = k.rowOut;
+    const uint16_t* gSh = k.shIdx;
+#pragma unroll
+    for (int j = 0; j < E; j++) {
+      const uint32_t p = min(tid + j * nt, lastP);
+      const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
+      const uint32_t rowO = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gOut) + ro * 4u);
+      const uint32_t sh = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const unsigned char*>(gSh) + p * 2u);
+      outOff[j] = (rowO + (p - ro * outCont)) * kScale;
+      shSlot[j] = sh * (uint32_t)sizeof(T);
+    }
+  };
+  T v[E];  // data on its way in: global memory -> registers -> LDS
+  auto issueLoads = [&](uint32_t offIn) __attribute__((always_inline)) {
+    const unsigned char* srcB = reinterpret_cast<const unsigned char*>(in + offIn);  // wave-uniform base
 #pragma unroll
     for (int j = 0; j < E; j++) {
       if (WIDE)
@@ -334,28 +343,65 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
       else
         v[j] = ldg<NT>(reinterpret_cast<const T*>(srcB + inOff[j]));
     }
-    __syncthreads();  // the previous item has finished reading the LDS buffer
-    {
-      // The slot of element p is p + (p >> padShift).  It is recomputed for every item from a
-      // value the compiler cannot see through, so that it does not park E more registers.
-      uint32_t tv = tid;
-      asm volatile("" : "+v"(tv));
+  };
+  // The slot of element p is p + (p >> padShift).  It is recomputed for every item from a value
+  // the compiler cannot see through, so that it does not park E more registers.
+  auto stage = [&]() __attribute__((always_inline)) {
+    uint32_t tv = tid;
+    asm volatile("" : "+v"(tv));
 #pragma unroll
-      for (int j = 0; j < E; j++) {
-        const uint32_t p = min(tv + j * nt, last);
-        *reinterpret_cast<T*>(ldsRaw + (p + (p >> padShift)) * (uint32_t)sizeof(T)) = v[j];
-      }
+    for (int j = 0; j < E; j++) {
+      const uint32_t p = min(tv + j * nt, last);
+      *reinterpret_cast<T*>(ldsRaw + (p + (p >> padShift)) * (uint32_t)sizeof(T)) = v[j];
     }
-    __syncthreads();
+  };
+  auto gatherAndStore = [&](uint32_t offOut) __attribute__((always_inline)) {
+    unsigned char* dstB = reinterpret_cast<unsigned char*>(out + offOut);
+    T u[E];
 #pragma unroll
-    for (int j = 0; j < E; j++) v[j] = *reinterpret_cast<const T*>(ldsRaw + shSlot[j]);
+    for (int j = 0; j < E; j++) u[j] = *reinterpret_cast<const T*>(ldsRaw + shSlot[j]);
 #pragma unroll
     for (int j = 0; j < E; j++) {
       if (WIDE)
-        stg<NT>(reinterpret_cast<T*>(dstB) + outOff[j], v[j]);
+        stg<NT>(reinterpret_cast<T*>(dstB) + outOff[j], u[j]);
       else
-        stg<NT>(reinterpret_cast<T*>(dstB + outOff[j]), v[j]);
+        stg<NT>(reinterpret_cast<T*>(dstB + outOff[j]), u[j]);
     }
+  };
+
+  // Software pipeline over the workgroup's items: the loads of item w+1 are issued before the LDS
+  // gather and the stores of item w, so they overlap, and the wait for them (the memory counter
+  // counts loads and stores in issue order) does not also wait for those stores to complete.
+  if (w0 >= w1) return;
+  uint32_t w = w0, offIn, offOut;
+  int cls;
+  locate(w, cls, offIn, offOut);
+  loadReadSide(cls);
+  issueLoads(offIn);
+  loadWriteSide(cls);  // after the data loads are out: its latency hides behind theirs
+  stage();
+  for (;;) {
+    if (w + 1 >= w1) {  // last item: nothing to fetch ahead
+      __syncthreads();
+      gatherAndStore(offOut);
+      break;
+    }
+    int clsNext;
+    uint32_t offInNext, offOutNext;
+    locate(w + 1, clsNext, offInNext, offOutNext);
+    // the slab class changes at most a few times per workgroup (wave-uniform tests)
+    if (clsNext != cls) loadReadSide(clsNext);
+    issueLoads(offInNext);
+    __syncthreads();  // item w is complete in the LDS buffer
+    gatherAndStore(offOut);
+    if (clsNext != cls) {
+      loadWriteSide(clsNext);
+      cls = clsNext;
+    }
+    __syncthreads();  // every lane has taken its elements of item w out of the buffer
+    stage();
+    w++;
+    offOut = offOutNext;
   }
 }
 
@@ -411,8 +457,8 @@ extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) { return pac
 // Registers per lane of packedKernel<T, E, *, WIDE> as compiled for gfx950 (the cache policy does
 // not change the count).  Rows: E = 1, 2, 4, 8, 16.
 extern "C" int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets) {
-  static const int narrow4[5] = {14, 22, 37, 67, 103}, wide4[5] = {17, 27, 47, 69, 128};
-  static const int narrow8[5] = {15, 23, 41, 73, 0}, wide8[5] = {18, 29, 51, 78, 0};
+  static const int narrow4[5] = {15, 23, 39, 68, 124}, wide4[5] = {18, 25, 40, 72, 128};
+  static const int narrow8[5] = {16, 25, 42, 80, 0}, wide8[5] = {18, 28, 48, 88, 0};
   int row = 0;
   while (row < 5 && (1 << row) != elemsPerThread) row++;
   if (row == 5 || (elemSize != 4 && elemSize != 8)) return 0;
