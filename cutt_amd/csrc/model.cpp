@@ -405,15 +405,15 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
   } else {
-    factor = 1.07 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
+    factor = 1.05 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
     // Sixteen elements per lane leave room for one workgroup per CU only; measured about 8 % slower
     // than the counters alone predict.
     if (plan.packed.elemsPerThread > 8) factor += 0.08;
     // Large items run faster than their counters say (fewer barriers and table loads per byte):
-    // measured 5-8 % between 4 KB and 64 KB of staged data.
-    factor -= 0.06 * (double)plan.ldsBytes / 65536.0;
+    // measured 5-10 % between 4 KB and 64 KB of staged data.
+    factor -= 0.10 * (double)plan.ldsBytes / 65536.0;
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);
