@@ -390,9 +390,13 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
       PlannerOptions v = base;
       v.tiledOrder = 3; v.superM = 16; v.superK = 16;   // square patches instead of strips
       variants.push_back(v);
-      v = base;
-      v.tiledOrder = 2;                                  // tiles along the output run fastest
-      variants.push_back(v);
+      for (int order : {1, 2}) {                         // rows of tiles along Mm / along Mk
+        const int cur = plans[best].method == kTiled ? plans[best].tiled.order : plans[best].tcopy.order;
+        if (order == cur) continue;
+        v = base;
+        v.tiledOrder = order;
+        variants.push_back(v);
+      }
     } else {
       for (int ipb : {1, 2, 4, 8}) {
         PlannerOptions v = base;
