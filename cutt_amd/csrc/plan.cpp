@@ -425,12 +425,14 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   if (opt.tiledOrder < 0) {
     // Measured over random shapes (forced Tiled, all orders timed):
     //  * with at most two tiles along Mk, plain rows of tiles along Mm (order 1) beat the strips by
-    //    6 % on average once there are many tiles along Mm;
+    //    6 % on average when there are some tens of tiles along Mm - but not thousands: the two
+    //    tiles that complete an output row must stay close (a 1528800 x 111 transpose ran at 3.4 TB/s
+    //    in rows and 5.4 TB/s in strips);
     //  * with two tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along
     //    Mk should run fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows
     //    are written as streams.
-    if (tilesK <= 2 && tilesM > opt.superM) o.order = 1;
-    else if (tilesM == 2 && tilesK >= 3 && volMmLastTile <= 24) o.order = 2;
+    if (tilesK <= 2 && tilesM > opt.superM && tilesM <= 64) o.order = 1;
+    else if (tilesM == 2 && tilesK >= 3 && tilesK <= 64 && volMmLastTile <= 24) o.order = 2;
   }
   // Super-tiles of up to superM x superK tiles, shrunk where a direction has fewer tiles.
   int64_t sm = std::min<int64_t>(opt.superM, tilesM), sk = std::min<int64_t>(opt.superK, tilesK);
