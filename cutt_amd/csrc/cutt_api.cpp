@@ -388,9 +388,9 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
     const PlannerOptions base = plannerOptions(force);
     if (plans[best].method == kTiled || plans[best].method == kTiledCopy) {
       PlannerOptions v = base;
-      v.tiledOrder = 3; v.superM = 16; v.superK = 16;   // square patches instead of strips
+      v.tiledOrder = 5; v.superM = 16; v.superK = 16;   // square patches instead of strips
       variants.push_back(v);
-      for (int order : {1, 2}) {                         // rows of tiles along Mm / along Mk
+      for (int order : {1, 2, 3, 5}) {                   // rows of tiles along Mm / along Mk, strips
         const int cur = plans[best].method == kTiled ? plans[best].tiled.order : plans[best].tcopy.order;
         if (order == cur) continue;
         v = base;

@@ -70,7 +70,9 @@ constexpr int kWaves = kTileThreads / 64;
 // sequence.  Orders 0-2 number the logical sequence with the Mbar position, the tile along Mm or
 // the tile along Mk running fastest; orders 3 and 4 visit the tiles in superM x superK super-tiles, so
 // that both the read neighbours (along Mm) and the write neighbours (along Mk) of a tile are
-// resident in the same L2 at about the same time.
+// resident in the same L2 at about the same time.  Order 5 is order 3 with the Mbar position running
+// between the super-tiles: the runs of consecutive Mbar positions, which are neighbours in memory
+// when the fastest Mbar rank follows Mk in the output (or Mm in the input), then meet in the L2 too.
 constexpr uint32_t kNumXcd = 8;
 
 struct TileOrder {
@@ -105,9 +107,16 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
   const uint32_t per = o.superM * o.superK;
   const uint32_t w = l % per;
   const uint32_t t = l / per;
-  const uint32_t st = t % (nSuperM * nSuperK);
-  m = t / (nSuperM * nSuperK);
-  if (o.order == 3) {  // inside a super-tile the tiles along Mm run fastest
+  uint32_t st;
+  if (o.order == 5) {  // like 3, but a super-tile is visited for every Mbar position in turn
+    st = t / volMbar;
+    m = t - st * volMbar;
+    if (st >= nSuperM * nSuperK) return false;
+  } else {
+    st = t % (nSuperM * nSuperK);
+    m = t / (nSuperM * nSuperK);
+  }
+  if (o.order != 4) {  // inside a super-tile the tiles along Mm run fastest
     tm = (st % nSuperM) * o.superM + (w % o.superM);
     tk = (st / nSuperM) * o.superK + (w / o.superM);
   } else {             // order 4: the tiles along Mk run fastest, super-tiles advance along Mk first
@@ -500,7 +509,7 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 4 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 5 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
@@ -531,7 +540,7 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 4 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 5 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))

@@ -339,8 +339,10 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double tilesK = copy ? plan.tcopy.tilesK : plan.tiled.tilesK;
     const double superM = copy ? plan.tcopy.superM : plan.tiled.superM;
     const Problem& pb = plan.pb;
+    const int order = copy ? plan.tcopy.order : plan.tiled.order;
     auto mbarDist = [&](int rank, bool input) -> double {
-      double d = tilesM * tilesK;
+      // order 5 walks the Mbar positions strip by strip, the others tensor slice by tensor slice
+      double d = order == 5 ? std::min(superM, tilesM) * tilesK : tilesM * tilesK;
       for (int k = 0; k < mb.n; k++) {
         const bool hit = input ? mb.d[k].strideIn == (uint32_t)pb.strideIn[rank]
                                : mb.d[k].strideOut == (uint32_t)pb.strideOut[rank];
@@ -404,6 +406,11 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double waste = 0.5 * (rdSlots + wrSlots) / (volMm * volMk) - 1.0;
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
+    // Tiny slabs of 4-byte elements: with one or two tiles along Mm and exactly two along Mk (a
+    // 65..128-long output run cut into a 256-byte piece and a remainder), 46 such plans among 3000
+    // random tensors ran 1.29-1.37 times (median) as long as predicted; every other class of tile
+    // counts stayed within 6 % of its prediction.
+    if (!copy && es == 4 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.3;
   } else {
     factor = 1.05 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +

@@ -421,19 +421,17 @@ struct TileOrdering {
 
 int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
                     int64_t volMmLastTile, TileOrdering& o) {
-  o.order = opt.tiledOrder >= 0 ? opt.tiledOrder : 3;
-  if (opt.tiledOrder < 0) {
-    // Measured over random shapes (forced Tiled, all orders timed):
-    //  * with at most two tiles along Mk, plain rows of tiles along Mm (order 1) beat the strips by
-    //    6 % on average when there are some tens of tiles along Mm - but not thousands: the two
-    //    tiles that complete an output row must stay close (a 1528800 x 111 transpose ran at 3.4 TB/s
-    //    in rows and 5.4 TB/s in strips);
-    //  * with two tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along
-    //    Mk should run fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows
-    //    are written as streams.
-    if (tilesK <= 2 && tilesM > opt.superM && tilesM <= 64) o.order = 1;
-    else if (tilesM == 2 && tilesK >= 3 && tilesK <= 64 && volMmLastTile <= 24) o.order = 2;
-  }
+  // Default: strips of super-tiles, each strip visited for all Mbar positions in turn (order 5;
+  // with one Mbar position that is order 3).  The runs of consecutive Mbar positions are usually
+  // neighbours in memory, so their shared lines meet in the L2: against finishing one Mbar position
+  // after the other, (192,270,27,110)/(3,2,0,1) fp64 went from 3.5 to 4.8 TB/s, C4's Tiled plan from
+  // 5.05 to 5.4 TB/s, and nothing measured got slower.
+  o.order = opt.tiledOrder >= 0 ? opt.tiledOrder : (volMbar > 1 ? 5 : 3);
+  // One measured exception (forced-Tiled sweep over random shapes, all orders timed): with two
+  // tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along Mk should run
+  // fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows are written as
+  // streams - as long as the two tiles that share an input row stay close (at most 64 tiles along Mk).
+  if (opt.tiledOrder < 0 && tilesM == 2 && tilesK >= 3 && tilesK <= 64 && volMmLastTile <= 24) o.order = 2;
   // Super-tiles of up to superM x superK tiles, shrunk where a direction has fewer tiles.
   int64_t sm = std::min<int64_t>(opt.superM, tilesM), sk = std::min<int64_t>(opt.superK, tilesK);
   // Equal-sized super-tiles: no nearly empty last one (its padding workgroups would leave XCDs idle).

@@ -46,18 +46,21 @@ def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk,
         m, tm = t // tiles_m, t % tiles_m
         ok = m < vol_mbar
     else:
-        assert order in (3, 4) and sup_m >= 1 and sup_k >= 1
+        assert order in (3, 4, 5) and sup_m >= 1 and sup_k >= 1
         n_sm, n_sk = -(-tiles_m // sup_m), -(-tiles_k // sup_k)
         per = sup_m * sup_k
         w, t = l % per, l // per
-        st, m = t % (n_sm * n_sk), t // (n_sm * n_sk)
-        if order == 3:
+        if order == 5:
+            st, m = t // vol_mbar, t % vol_mbar
+        else:
+            st, m = t % (n_sm * n_sk), t // (n_sm * n_sk)
+        if order != 4:
             tm = (st % n_sm) * sup_m + w % sup_m
             tk = (st // n_sm) * sup_k + w // sup_m
         else:
             tk = (st % n_sk) * sup_k + w % sup_k
             tm = (st // n_sk) * sup_m + w // sup_k
-        ok = (m < vol_mbar) & (tm < tiles_m) & (tk < tiles_k)
+        ok = (m < vol_mbar) & (st < n_sm * n_sk) & (tm < tiles_m) & (tk < tiles_k)
     key = (m[ok] * tiles_k + tk[ok]) * tiles_m + tm[ok]
     assert key.size == tiles_m * tiles_k * vol_mbar, "tile decode misses or repeats tiles"
     assert np.array_equal(np.sort(key), np.arange(key.size))
