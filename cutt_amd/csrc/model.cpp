@@ -405,14 +405,14 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double wrSlots = copy ? rdSlots : rows16(volMm) * tilesK * kTile;
     const double waste = 0.5 * (rdSlots + wrSlots) / (volMm * volMk) - 1.0;
     factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
-             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? 0.10 : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
+             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? (es == 4 ? 0.20 : 0.10) : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
     // Tiny slabs of 4-byte elements: with one or two tiles along Mm and exactly two along Mk (a
     // 65..128-long output run cut into a 256-byte piece and a remainder), 46 such plans among 3000
     // random tensors ran 1.29-1.37 times (median) as long as predicted; every other class of tile
     // counts stayed within 6 % of its prediction.
     if (!copy && es == 4 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.3;
   } else {
-    factor = 1.05 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial + (es == 4 ? 0.038 : 0.0) -
+    factor = 1.05 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.03 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
     // Sixteen elements per lane leave room for one workgroup per CU only; measured about 8 % slower
