@@ -382,64 +382,74 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
       p.release();
     }
   }
-  // Second stage: variants of the winner that differ only in workgroup ordering and granularity.
+  // Second stage: the winner's launch geometry is tuned one knob at a time (tile order, work items
+  // per workgroup, order of the Mbar ranks, cache policy); a setting that measures faster is kept
+  // for the knobs that follow.
   if (!failed && best >= 0 && plans[best].method != kTrivial) {
-    std::vector<PlannerOptions> variants;
-    const PlannerOptions base = plannerOptions(force);
-    if (plans[best].method == kTiled || plans[best].method == kTiledCopy) {
-      PlannerOptions v = base;
-      v.tiledOrder = 5; v.superM = 16; v.superK = 16;   // square patches instead of strips
-      variants.push_back(v);
-      for (int order : {1, 2, 3, 5}) {                   // rows of tiles along Mm / along Mk, strips
-        const int cur = plans[best].method == kTiled ? plans[best].tiled.order : plans[best].tcopy.order;
-        if (order == cur) continue;
-        v = base;
-        v.tiledOrder = order;
-        variants.push_back(v);
+    const bool tiled = plans[best].method == kTiled || plans[best].method == kTiledCopy;
+    // options that reproduce the winner as it stands
+    PlannerOptions cur = plannerOptions(force);
+    cur.cachePolicy = cachePolicyOf(plans[best]);
+    if (tiled) cur.tiledOrder = plans[best].method == kTiled ? plans[best].tiled.order : plans[best].tcopy.order;
+    else cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
+    const PlannerOptions start = cur;
+
+    // Tries `v`; keeps it (and returns true) if it is faster than the best so far.
+    auto tryVariant = [&](const PlannerOptions& v, bool sameGridIsSamePlan) -> bool {
+      Plan q;
+      if (!rebuildPlan(plans[best], props, v, q)) return false;
+      if (sameGridIsSamePlan && q.numBlocks == plans[best].numBlocks) return false;
+      setCachePolicy(q, v.cachePolicy);
+      if (!estimatePlan(q, props, 10)) return false;
+      double t;
+      if (!timePlan(q, t)) { failed = true; return false; }
+      if (t >= bestUs) return false;
+      bestUs = t;
+      us.push_back(t);
+      plans[best].release();
+      plans.push_back(std::move(q));
+      best = (int)plans.size() - 1;
+      return true;
+    };
+
+    if (tiled) {
+      // square patches instead of strips, rows of tiles along Mm / along Mk, strips per Mbar
+      // position / for all Mbar positions in turn
+      struct TileKnob { int order, superM, superK; };
+      for (const TileKnob& k : {TileKnob{5, 16, 16}, TileKnob{1, start.superM, start.superK},
+                                TileKnob{2, start.superM, start.superK}, TileKnob{3, start.superM, start.superK},
+                                TileKnob{5, start.superM, start.superK}}) {
+        if (failed) break;
+        if (k.order == start.tiledOrder && k.superM == start.superM) continue;
+        PlannerOptions v = cur;
+        v.tiledOrder = k.order; v.superM = k.superM; v.superK = k.superK;
+        if (tryVariant(v, false)) cur = v;
       }
     } else {
       for (int ipb : {1, 2, 4, 8}) {
-        PlannerOptions v = base;
-        if (ipb == plans[best].packed.itemsPerBlock) continue;
+        if (failed) break;
+        if (ipb == start.maxItemsPerBlock) continue;
+        PlannerOptions v = cur;
         v.maxItemsPerBlock = ipb;
-        variants.push_back(v);
+        if (tryVariant(v, true)) cur = v;
       }
-      // the order in which consecutive work items walk the Mbar ranks decides which partly used
-      // lines neighbouring workgroups share in the L2; it can move the time by 20 %
-      for (int order : {0, 1, 2}) {
-        if (order == base.mbarOrder || std::getenv("CUTT_MBAR_ORDER")) continue;
-        PlannerOptions v = base;
-        v.mbarOrder = order;
-        v.orderOnly = true;
-        variants.push_back(v);
-      }
+    }
+    // the order in which consecutive work items (or strips of tiles) walk the Mbar ranks decides
+    // which partly used lines neighbouring workgroups share in the L2; it can move the time by 20 %
+    for (int order : {0, 1, 2}) {
+      if (failed || std::getenv("CUTT_MBAR_ORDER")) break;
+      if (order == start.mbarOrder) continue;
+      PlannerOptions v = cur;
+      v.mbarOrder = order;
+      if (tryVariant(v, false)) cur = v;
     }
     // ... and the other cache policies of the global accesses
-    const int curPolicy = cachePolicyOf(plans[best]);
     for (int pol : {0, 1, 3}) {
-      if (pol == curPolicy || std::getenv("CUTT_CACHE_POLICY")) continue;
-      PlannerOptions v = base;
+      if (failed || std::getenv("CUTT_CACHE_POLICY")) break;
+      if (pol == start.cachePolicy) continue;
+      PlannerOptions v = cur;
       v.cachePolicy = pol;
-      v.policyOnly = true;
-      variants.push_back(v);
-    }
-    for (const PlannerOptions& v : variants) {
-      Plan q;
-      if (!rebuildPlan(plans[best], props, v, q)) continue;
-      if (!v.policyOnly) {
-        if (!v.orderOnly && q.numBlocks == plans[best].numBlocks && q.method != kTiled && q.method != kTiledCopy) continue;
-        setCachePolicy(q, curPolicy);
-      }
-      if (!estimatePlan(q, props, 10)) continue;
-      double t;
-      if (!timePlan(q, t)) { failed = true; break; }
-      if (t < bestUs) {
-        bestUs = t;
-        us.push_back(t);
-        plans[best].release();
-        plans.push_back(std::move(q));
-        best = (int)plans.size() - 1;
-      }
+      if (tryVariant(v, false)) cur = v;
     }
   }
   cuttHipEventDestroy(evStart);

@@ -132,9 +132,7 @@ struct PlannerOptions {
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
   int maxItemsPerBlock = 0;  // Packed/PackedSplit: work items one workgroup handles at most; 0 = by item size
-  bool policyOnly = false;  // (measuring planner) this variant differs only in the cache policy
   int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores
-  bool orderOnly = false;   // (measuring planner) this variant differs only in the order of the Mbar ranks
   int mbarOrder = 2;        // order of the Mbar ranks: 0 = input order, 1 = output order,
                             // 2 = first input rank outside Mmk, then output order
   bool wideOffsets = false; // Packed/PackedSplit: 64-bit address arithmetic also below 4 GB (tests)
