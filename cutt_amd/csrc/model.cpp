@@ -412,7 +412,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // counts stayed within 6 % of its prediction.
     if (!copy && es == 4 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.3;
   } else {
-    factor = 1.05 + 0.093 * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.03 : 0.0) -
+    factor = 1.05 + (es == 4 ? 0.17 : 0.093) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
     // Sixteen elements per lane leave room for one workgroup per CU only; measured about 8 % slower
