@@ -413,10 +413,12 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
     };
 
     if (tiled) {
-      // square patches instead of strips, rows of tiles along Mm / along Mk, strips per Mbar
-      // position / for all Mbar positions in turn
+      // patches of several shapes instead of strips (small patches walked for all Mbar positions in
+      // turn make long sequential streams of a batched 2-D transpose: C2 +4...7 %), rows of tiles
+      // along Mm / along Mk, strips per Mbar position / for all Mbar positions in turn
       struct TileKnob { int order, superM, superK; };
-      for (const TileKnob& k : {TileKnob{5, 16, 16}, TileKnob{1, start.superM, start.superK},
+      for (const TileKnob& k : {TileKnob{5, 16, 16}, TileKnob{5, 2, 8}, TileKnob{5, 8, 2}, TileKnob{5, 32, 2},
+                                TileKnob{1, start.superM, start.superK},
                                 TileKnob{2, start.superM, start.superK}, TileKnob{3, start.superM, start.superK},
                                 TileKnob{5, start.superM, start.superK}}) {
         if (failed) break;
