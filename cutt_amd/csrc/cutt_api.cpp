@@ -11,12 +11,15 @@
  * because a first launch also pays for loading the kernel.
  */
 #include <algorithm>
+#include <atomic>
 #include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
 #include <string>
+#include <system_error>
+#include <thread>
 #include <unordered_map>
 #include <vector>
 
@@ -180,6 +183,41 @@ void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
   setCachePolicy(p, wholeReads ? (wholeWrites ? 3 : 1) : 0);
 }
 
+// Runs f(0) .. f(n-1) on up to eight host threads (CUTT_PLAN_THREADS caps the number; 1 = the
+// calling thread only) and returns when all have finished.  The calls must not depend on each
+// other: the model's estimate of a candidate is a pure function of that candidate, so a plan does
+// not depend on the number of threads.
+template <class F>
+void parallelFor(int n, F&& f) {
+  int cap = 8;
+  if (const char* e = std::getenv("CUTT_PLAN_THREADS")) cap = std::max(1, std::atoi(e));
+  const unsigned hw = std::thread::hardware_concurrency();
+  const int nt = std::min({n, cap, hw ? (int)hw : 1});
+  std::atomic<int> next{0};
+  auto work = [&]() {
+    for (int i = next.fetch_add(1); i < n; i = next.fetch_add(1)) f(i);
+  };
+  std::vector<std::thread> helpers;
+  for (int t = 1; t < nt; t++) {
+    try {
+      helpers.emplace_back(work);
+    } catch (const std::system_error&) {
+      break;  // no more threads to be had: the calling thread does the rest
+    }
+  }
+  work();
+  for (std::thread& t : helpers) t.join();
+}
+
+// Model estimate of every candidate; false if one of them fails.
+bool estimateAll(std::vector<Plan>& plans, const cuttHipDeviceProps& props) {
+  std::atomic<bool> ok{true};
+  parallelFor((int)plans.size(), [&](int i) {
+    if (!estimatePlan(plans[i], props, 10)) ok = false;
+  });
+  return ok;
+}
+
 PlannerOptions plannerOptions(int forceMethod);
 
 // The order in which consecutive work items walk the Mbar ranks decides whether the lines shared
@@ -194,16 +232,24 @@ void refineMbarOrder(std::vector<Plan>& plans, const cuttHipDeviceProps& props, 
     if (plans[i].method != kTrivial) idx.push_back(i);
   std::sort(idx.begin(), idx.end(),
             [&](int a, int b) { return plans[a].model.usPredicted < plans[b].model.usPredicted; });
-  for (size_t k = 0; k < idx.size() && k < 3; k++) {
-    Plan& p = plans[idx[k]];
-    for (int order : {0, 1, 2}) {
-      if (order == base.mbarOrder) continue;
-      PlannerOptions opt = base;
-      opt.mbarOrder = order;
-      Plan q;
-      if (!rebuildPlan(p, props, opt, q) || !estimatePlan(q, props, 10)) continue;
-      if (q.model.usPredicted < p.model.usPredicted) p = std::move(q);
-    }
+  struct Trial {
+    int plan, order;
+    bool ok;
+    Plan q;
+  };
+  std::vector<Trial> trials;
+  for (size_t k = 0; k < idx.size() && k < 3; k++)
+    for (int order : {0, 1, 2})
+      if (order != base.mbarOrder) trials.push_back({idx[k], order, false, Plan()});
+  parallelFor((int)trials.size(), [&](int i) {
+    Trial& t = trials[i];
+    PlannerOptions opt = base;
+    opt.mbarOrder = t.order;
+    t.ok = rebuildPlan(plans[t.plan], props, opt, t.q) && estimatePlan(t.q, props, 10);
+  });
+  for (Trial& t : trials) {
+    Plan& p = plans[t.plan];
+    if (t.ok && t.q.model.usPredicted < p.model.usPredicted) p = std::move(t.q);
   }
 }
 
@@ -293,8 +339,7 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
   }
   std::vector<Plan> plans;
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
-  for (Plan& p : plans)
-    if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
+  if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
   refineMbarOrder(plans, props, force);
   const int best = chooseHeuristic(plans);
   if (best < 0) return CUTT_INTERNAL_ERROR;
@@ -321,10 +366,8 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   std::vector<Plan> plans;
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
   if (plans.empty()) return CUTT_INTERNAL_ERROR;
-  for (Plan& p : plans) {
-    if (!estimatePlan(p, props, 10)) return CUTT_INTERNAL_ERROR;
-    chooseCachePolicy(p, props);
-  }
+  if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
+  for (Plan& p : plans) chooseCachePolicy(p, props);
 
   size_t numBytes = sizeofType;
   for (int i = 0; i < rank; i++) numBytes *= (size_t)dim[i];
@@ -586,11 +629,9 @@ extern "C" void* cuttCandidatesCreateEx(int rank, const int* dim, const int* per
     delete l;
     return nullptr;
   }
-  for (Plan& p : l->plans) {
-    if (!p.buildTables() || !estimatePlan(p, props, 10)) {
-      delete l;
-      return nullptr;
-    }
+  if (!estimateAll(l->plans, props)) {
+    delete l;
+    return nullptr;
   }
   l->best = chooseHeuristic(l->plans);
   return l;

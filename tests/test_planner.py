@@ -153,3 +153,18 @@ def test_plans_are_deterministic(cutt):
     a = method_set(cutt, (31, 549, 2, 3), (3, 0, 2, 1), 8)
     b = method_set(cutt, (31, 549, 2, 3), (3, 0, 2, 1), 8)
     assert [i.as_dict() for i in a[0]] == [i.as_dict() for i in b[0]]
+
+
+def test_plans_do_not_depend_on_the_number_of_planner_threads(cutt, monkeypatch):
+    # The candidates are estimated on several host threads; each estimate is a pure function of
+    # its candidate, so the list and the pick are those of the single-threaded planner.
+    cases = [((30, 3, 20, 9, 24, 29, 15), (5, 2, 6, 4, 0, 1, 3), 4),
+             ((25, 20, 4, 30, 8, 13, 40), (0, 2, 1, 5, 6, 3, 4), 8),
+             ((1024, 64, 1024, 3), (2, 1, 0, 3), 8)]
+    for dim, perm, es in cases:
+        got = []
+        for threads in ("1", "3", "8"):
+            monkeypatch.setenv("CUTT_PLAN_THREADS", threads)
+            infos, best = method_set(cutt, dim, perm, es)
+            got.append(([i.as_dict() for i in infos], best.as_dict()))
+        assert got[0] == got[1] == got[2]
