@@ -32,6 +32,8 @@
  */
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+
 #include "hip_layer.h"
 #include "mbar_decode.h"
 
@@ -570,8 +572,9 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
 // Called when a packed plan is activated (so that a plan's first cuttExecute already is a plain
 // kernel launch) and, as a cheap check, before every launch.
 extern "C" int cuttHipPreparePacked(void) {
-  // Function attributes are kept per device; benign if two threads race: the calls are idempotent.
-  static bool ldsOptInDone[64] = {};
+  // Function attributes are kept per device.  Two threads may both find the flag clear and both
+  // make the calls: they are idempotent.
+  static std::atomic<bool> ldsOptInDone[64];
   int dev = 0;
   if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
   const bool tracked = dev >= 0 && dev < 64;

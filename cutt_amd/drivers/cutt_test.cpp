@@ -14,12 +14,18 @@
  *   5  the cost model's transaction counters against brute force
  *      (reference test5, :410-431)
  *   6  what the API refuses, and that the checker notices a wrong element
+ *   7  four host threads that plan, execute, check and destroy at the same time
+ *      (the reference keeps its plans in an unguarded table, src/cutt.cpp:35-39; this
+ *      library guards its own)
  * Prints "test OK" or "test FAIL"; the exit status says the same.
  */
 #include <algorithm>
+#include <atomic>
 #include <cstring>
+#include <mutex>
 #include <set>
 #include <string>
+#include <thread>
 
 #include "cutt_ext.h"
 #include "driver_util.h"
@@ -321,6 +327,65 @@ bool test6() {
   return true;
 }
 
+// Four host threads, each with a stream, a checker and a quarter of the output buffer of its own,
+// plan (every third tensor with cuttPlanMeasure), execute, check and destroy seeded random tensors
+// at the same time.  The input buffer is shared and only read.
+bool test7(uint64_t seed) {
+  const int numThreads = 4, tensorsPerThread = 12;
+  const size_t sliceBytes = (size_t)kDataElems * 8 / numThreads;
+  std::atomic<int> failures{0};
+  std::atomic<long long> done{0};
+  std::mutex printMutex;
+  auto fail = [&](int t, const char* what, const std::vector<int>& dim, const std::vector<int>& perm, size_t es) {
+    std::lock_guard<std::mutex> lock(printMutex);
+    std::printf("test7: thread %d: %s, elemsize %zu\n", t, what, es);
+    printVec("  dimensions ", dim);
+    printVec("  permutation", perm);
+    failures++;
+  };
+  auto worker = [&](int t) {
+    Rng rng(seed * 7919 + (uint64_t)t);
+    TensorChecker mine;
+    hipStream_t stream;
+    if (hipStreamCreate(&stream) != hipSuccess) {
+      failures++;
+      return;
+    }
+    char* out = (char*)dataOut + (size_t)t * sliceBytes;
+    for (int i = 0; i < tensorsPerThread && failures == 0; i++) {
+      const int rank = 2 + rng.below(6);
+      const size_t es = (i + t) % 2 ? 4 : 8;
+      std::vector<int> dim, perm(rank);
+      for (int r = 0; r < rank; r++) perm[r] = r;
+      const double vol = std::max(std::pow(3.0, rank), 1e4 + 4e6 * rng.uniform());
+      if (!randomDims(rng, vol, rank, 0.3, dim) || (size_t)volumeOf(dim) * es > sliceBytes) continue;
+      rng.shuffle(perm);
+      cuttHandle plan = 0;
+      cuttResult r = i % 3 == 2 ? cuttPlanMeasure(&plan, rank, dim.data(), perm.data(), es, stream, dataIn, out)
+                                : cuttPlan(&plan, rank, dim.data(), perm.data(), es, stream);
+      if (r != CUTT_SUCCESS) {
+        fail(t, "plan refused", dim, perm, es);
+        break;
+      }
+      bool ok = hipMemsetAsync(out, 0xff, (size_t)volumeOf(dim) * es, stream) == hipSuccess;
+      ok = ok && cuttExecute(plan, dataIn, out) == CUTT_SUCCESS;
+      ok = ok && hipStreamSynchronize(stream) == hipSuccess;
+      if (!ok) fail(t, "execute failed", dim, perm, es);
+      else if (mine.check(rank, dim.data(), perm.data(), es, out).numWrong != 0) fail(t, "wrong result", dim, perm, es);
+      if (cuttDestroy(plan) != CUTT_SUCCESS) fail(t, "destroy refused", dim, perm, es);
+      done++;
+    }
+    (void)hipStreamDestroy(stream);
+  };
+  HIP_CHECK(hipDeviceSynchronize());
+  std::vector<std::thread> threads;
+  for (int t = 0; t < numThreads; t++) threads.emplace_back(worker, t);
+  for (std::thread& th : threads) th.join();
+  HIP_CHECK(hipDeviceSynchronize());
+  numTensors += done;
+  return failures == 0 && done > 0;
+}
+
 void usage() {
   std::printf("cutt_test [options]\n");
   std::printf("Options:\n");
@@ -337,7 +402,7 @@ void usage() {
 int main(int argc, char* argv[]) {
   int gpuid = -1, samples = 100;
   uint64_t seed = 1;
-  std::set<int> tests = {1, 2, 3, 4, 5, 6};
+  std::set<int> tests = {1, 2, 3, 4, 5, 6, 7};
   for (int i = 1; i < argc; i++) {
     std::string a = argv[i];
     if (a == "-device" && i + 1 < argc) {
@@ -373,7 +438,8 @@ int main(int argc, char* argv[]) {
     const char* what;
   };
   const Entry entries[] = {{1, "all permutations, ranks 2-7"}, {2, "random tensors, ranks 2-15"}, {3, "hand-picked shapes"},
-                           {4, "ten streams"},                 {5, "model counters"},             {6, "refusals and checker"}};
+                           {4, "ten streams"},                 {5, "model counters"},             {6, "refusals and checker"},
+                           {7, "four host threads"}};
   for (const Entry& e : entries) {
     if (!ok || !tests.count(e.id)) continue;
     std::printf("test %d: %s\n", e.id, e.what);
@@ -385,6 +451,7 @@ int main(int argc, char* argv[]) {
       case 4: ok = test4(); break;
       case 5: ok = test5(seed); break;
       case 6: ok = test6(); break;
+      case 7: ok = test7(seed); break;
     }
     std::printf("test %d %s\n", e.id, ok ? "passed" : "FAILED");
     std::fflush(stdout);
