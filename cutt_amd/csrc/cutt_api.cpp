@@ -156,7 +156,6 @@ int cachePolicyOf(const Plan& p) {
 // (Not applied when CUTT_CACHE_POLICY pins the policy.)
 void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
   if (std::getenv("CUTT_CACHE_POLICY")) return;
-  if (p.method == kTrivial) return;
   // The memory-side cache decides for small and medium tensors (measured on random tensors of
   // 4M-200M elements): while input and output fit it together, ordinary accesses are best
   // (non-temporal ones go past it: 65-72 % of memcpy instead of 80-89 %); up to about 3.5 times

@@ -218,6 +218,8 @@ const char* cuttHipErrorString(int err);
 int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);
+/* Plain copy of `bytes` bytes (a multiple of 4) for the Trivial method; cachePolicy as above. */
+int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int cachePolicy, void* stream);
 /* One-time kernel attribute setup of the packed kernels on the current device (idempotent). */
 int cuttHipPreparePacked(void);
 

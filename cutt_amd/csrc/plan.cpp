@@ -520,15 +520,17 @@ bool allowed(const PlannerOptions& opt, int method) {
   return opt.forceMethod == 0 || opt.forceMethod == method;
 }
 
-void addTrivial(const Problem& red, std::vector<Plan>& plans) {
+void addTrivial(const Problem& red, const PlannerOptions& opt, std::vector<Plan>& plans) {
   Plan p;
   p.method = kTrivial;
   p.pb = red;
   p.fromReduced = true;
   p.split.method = kTrivial;
   p.split.update(1, 1, red);
-  p.numBlocks = 1;
-  p.numThreads = 1;
+  // one 4-KB piece per workgroup (hip_layer: cuttHipLaunchCopy)
+  p.numBlocks = std::max<int64_t>(1, (red.volume * red.elemSize / 16 + 255) / 256);
+  p.numThreads = 256;
+  p.packed.cachePolicy = opt.cachePolicy;  // where a Trivial plan keeps its policy
   plans.push_back(std::move(p));
 }
 
@@ -727,7 +729,7 @@ bool createPlans(const Problem& orig, const Problem& red, const cuttHipDevicePro
   if (identity) {
     // Everything fuses into one rank (or would, if the fused extent still fitted an int): a plain
     // copy is the only candidate.
-    addTrivial(red, plans);
+    addTrivial(red, opt, plans);
     return true;
   }
   addTiled(red, props, opt, plans);
@@ -840,7 +842,7 @@ int Plan::activate() {
 int Plan::launch(const void* in, void* out) {
   switch (method) {
     case kTrivial:
-      return cuttHipMemcpyDtoDAsync(out, in, (size_t)pb.volume * pb.elemSize, stream);
+      return cuttHipLaunchCopy(in, out, (size_t)pb.volume * pb.elemSize, packed.cachePolicy, stream);
     case kTiled:
       return cuttHipLaunchTiled(&tiled, in, out, stream);
     case kTiledCopy:

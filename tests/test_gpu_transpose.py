@@ -328,3 +328,42 @@ def test_identity_of_2_to_31_elements_is_a_copy(gpu):
     torch.cuda.synchronize()
     assert torch.equal(a, b)
     assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+
+
+def test_trivial_copy_sizes_alignments_and_cache_policies(gpu):
+    # The Trivial method is a kernel of the library (16 bytes per lane), not the runtime's copy:
+    # byte counts that are not multiples of 16, buffers that start off the 16-byte grid (those go
+    # to the runtime's copy), each cache policy (chosen by size), and the words after the copied
+    # range must stay untouched.
+    import torch
+    import cutt_amd as cutt
+    st = gpu.stream_handle()
+    cases = [((3, 3), 4), ((3, 5, 7), 4), ((2, 2), 4), ((2, 2), 8), ((3, 5, 7), 8), ((1023, 5), 4),
+             ((1025, 1023), 4), ((4099, 4001), 8),            # 131 MB: ordinary accesses
+             ((8193, 8191), 8),                               # 537 MB: streaming loads
+             ((16385, 8191), 8)]                              # 1.07 GB: streaming loads and stores
+    policies = set()
+    for dim, es in cases:
+        n = int(np.prod(dim))
+        words = n * es // 4
+        perm = tuple(range(len(dim)))
+        rc, h = cutt.cuttPlan(len(dim), dim, perm, es, st)
+        assert rc == cutt.CUTT_SUCCESS
+        info = cutt.get_plan_info(h)
+        assert info.method_name == "Trivial"
+        policies.add(info.cachePolicy)
+        for shift_in, shift_out in ((0, 0), (1, 0), (0, 2), (3, 3)):   # in 4-byte words
+            if es == 8 and (shift_in % 2 or shift_out % 2):
+                continue
+            say("trivial dim=%s es=%d shifts=%d,%d policy=%d" % (dim, es, shift_in, shift_out, info.cachePolicy))
+            a = torch.empty(words + 8, dtype=torch.int32, device="cuda")
+            a.random_()
+            b = torch.full((words + 8,), -1, dtype=torch.int32, device="cuda")
+            src, dst = a[shift_in:shift_in + words], b[shift_out:shift_out + words]
+            assert cutt.cuttExecute(h, src.data_ptr(), dst.data_ptr()) == cutt.CUTT_SUCCESS
+            torch.cuda.synchronize()
+            assert torch.equal(src, dst)
+            assert bool((b[:shift_out] == -1).all()) and bool((b[shift_out + words:] == -1).all())
+            del a, b
+        assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+    assert policies == {0, 1, 3}
