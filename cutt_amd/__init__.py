@@ -11,6 +11,6 @@ from .api import (  # noqa: F401
     METHOD_NAMES, METHOD_TRIVIAL, METHOD_PACKED, METHOD_PACKEDSPLIT, METHOD_TILED, METHOD_TILEDCOPY,
     CuttError, PlanInfo, lib, lib_path,
     cuttPlan, cuttPlanMeasure, cuttPlanFromCandidate, cuttExecute, cuttDestroy,
-    get_plan_info, set_method_override, get_last_measurement, reduce_ranks, Candidates,
+    get_plan_info, set_method_override, clear_plan_cache, get_last_measurement, reduce_ranks, Candidates,
 )
 from .build import build  # noqa: F401

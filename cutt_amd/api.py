@@ -100,6 +100,8 @@ def lib():
     l.cuttSetMethodOverride.restype = None
     l.cuttGetMethodOverride.argtypes = []
     l.cuttGetMethodOverride.restype = ctypes.c_int
+    l.cuttClearPlanCache.argtypes = []
+    l.cuttClearPlanCache.restype = None
     l.cuttGetLastMeasurement.argtypes = [ctypes.POINTER(PlanInfo), ctypes.c_int]
     l.cuttGetLastMeasurement.restype = ctypes.c_int
     l.cuttReduceRanks.argtypes = [ctypes.c_int, ip, ip, ip, ip]
@@ -182,6 +184,10 @@ def get_plan_info(handle):
 
 def set_method_override(method):
     lib().cuttSetMethodOverride(int(method))
+
+
+def clear_plan_cache():
+    lib().cuttClearPlanCache()
 
 
 def get_last_measurement():

@@ -16,6 +16,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <list>
 #include <mutex>
 #include <string>
 #include <system_error>
@@ -45,6 +46,66 @@ cuttHandle gNextHandle = 0;
 std::unordered_map<int, cuttHipDeviceProps> gDeviceProps;
 int gMethodOverride = -1;  // -1 = not initialised from the environment yet
 std::vector<cuttPlanInfo> gLastMeasurement;
+
+// What cuttPlan decided for the problems it saw last, most recent first: a second cuttPlan for the
+// same tensor on the same device copies the decision instead of enumerating and estimating the
+// candidates again.  Entries hold host data only (no device tables, no stream).
+struct CachedDecision {
+  std::string key;
+  Plan plan;
+  int numCandidates;
+};
+std::list<CachedDecision> gDecisions;
+std::unordered_map<std::string, std::list<CachedDecision>::iterator> gDecisionIndex;
+
+// Entries the cache may hold: CUTT_PLAN_CACHE (default 64; 0 switches it off).
+size_t planCacheCapacity() {
+  if (const char* e = std::getenv("CUTT_PLAN_CACHE")) return (size_t)std::max(0, std::atoi(e));
+  return 64;
+}
+
+// Everything a decision depends on: device, method override, the tensor, and the tuning variables
+// of the environment as they are now.
+std::string planKey(int deviceID, int force, int rank, const int* dim, const int* perm, size_t sizeofType) {
+  std::string k;
+  auto put = [&](long long v) {
+    k += std::to_string(v);
+    k += ',';
+  };
+  put(deviceID); put(force); put((long long)sizeofType); put(rank);
+  for (int i = 0; i < rank; i++) put(dim[i]);
+  for (int i = 0; i < rank; i++) put(perm[i]);
+  for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
+                           "CUTT_MAX_ITEMS", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
+                           "CUTT_SUPER_M", "CUTT_SUPER_K"}) {
+    const char* e = std::getenv(name);
+    k += e ? e : "-";
+    k += ';';
+  }
+  return k;
+}
+
+bool planCacheLookup(const std::string& key, Plan& out, int& numCandidates) {
+  std::lock_guard<std::mutex> lock(gMutex);
+  auto it = gDecisionIndex.find(key);
+  if (it == gDecisionIndex.end()) return false;
+  gDecisions.splice(gDecisions.begin(), gDecisions, it->second);  // most recent first
+  out = it->second->plan.clone();
+  numCandidates = it->second->numCandidates;
+  return true;
+}
+
+void planCacheInsert(const std::string& key, const Plan& chosen, int numCandidates) {
+  const size_t capacity = planCacheCapacity();
+  std::lock_guard<std::mutex> lock(gMutex);
+  if (capacity == 0 || gDecisionIndex.count(key)) return;
+  gDecisions.push_front(CachedDecision{key, chosen.clone(), numCandidates});
+  gDecisionIndex[key] = gDecisions.begin();
+  while (gDecisions.size() > capacity) {
+    gDecisionIndex.erase(gDecisions.back().key);
+    gDecisions.pop_back();
+  }
+}
 
 int methodOverrideLocked() {
   if (gMethodOverride < 0) {
@@ -336,6 +397,14 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
     std::lock_guard<std::mutex> lock(gMutex);
     force = methodOverrideLocked();
   }
+  const bool useCache = planCacheCapacity() > 0;
+  const std::string key = useCache ? planKey(deviceID, force, rank, dim, permutation, sizeofType) : std::string();
+  if (useCache) {
+    Plan known;
+    int numCandidates = 0;
+    if (planCacheLookup(key, known, numCandidates))
+      return storePlan(handle, std::move(known), (void*)stream, deviceID, numCandidates, 0.0, t0);
+  }
   std::vector<Plan> plans;
   if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
   if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
@@ -343,6 +412,7 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
   const int best = chooseHeuristic(plans);
   if (best < 0) return CUTT_INTERNAL_ERROR;
   chooseCachePolicy(plans[best], props);
+  if (useCache) planCacheInsert(key, plans[best], (int)plans.size());
   return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
 }
 
@@ -612,6 +682,12 @@ struct CandidateList {
   int best = -1;
 };
 }  // namespace
+
+extern "C" void cuttClearPlanCache(void) {
+  std::lock_guard<std::mutex> lock(gMutex);
+  gDecisionIndex.clear();
+  gDecisions.clear();
+}
 
 extern "C" void* cuttCandidatesCreateEx(int rank, const int* dim, const int* permutation,
                                         size_t sizeofType, size_t ldsPerBlock) {

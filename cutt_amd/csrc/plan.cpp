@@ -201,6 +201,31 @@ Plan& Plan::operator=(Plan&& o) noexcept {
   return *this;
 }
 
+Plan Plan::clone() const {
+  Plan q;
+  q.method = method;
+  q.split = split;
+  q.pb = pb;
+  q.fromReduced = fromReduced;
+  q.deviceID = deviceID;
+  q.stream = stream;
+  q.tiled = tiled;
+  q.tcopy = tcopy;
+  q.packed = packed;
+  for (int c = 0; c < 4; c++) {  // device tables stay with the original
+    q.packed.cls[c].rowIn = nullptr;
+    q.packed.cls[c].rowOut = nullptr;
+    q.packed.cls[c].shIdx = nullptr;
+  }
+  q.ldsBytes = ldsBytes;
+  q.numBlocks = numBlocks;
+  q.numThreads = numThreads;
+  for (int c = 0; c < 4; c++) q.tab[c] = tab[c];
+  q.tablesBuilt = tablesBuilt;
+  q.model = model;
+  return q;
+}
+
 void Plan::release() {
   if (dTables) {
     cuttHipFree(dTables);

@@ -118,6 +118,7 @@ struct Plan {
   Plan(Plan&& o) noexcept;
   Plan& operator=(Plan&& o) noexcept;
 
+  Plan clone() const;             // host-side copy of a plan that has no device tables yet
   bool buildTables();             // Packed/PackedSplit: fill tab[]; others: no-op
   int activate();                 // upload tables; returns 0 or a HIP error code
   int launch(const void* in, void* out);  // asynchronous on stream

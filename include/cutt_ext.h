@@ -71,6 +71,17 @@ void cuttSetMethodOverride(int method);
 int cuttGetMethodOverride(void);
 
 /*
+ * cuttPlan remembers what it decided for the tensors it planned last (per
+ * device, method override and tuning environment; 64 entries, least recently
+ * used dropped first; CUTT_PLAN_CACHE = n changes the number, 0 switches the
+ * memory off), so that planning the same tensor again skips the enumeration
+ * and the cost model.  Every plan still owns its device tables and its stream.
+ * cuttPlanMeasure neither reads nor fills this memory.  The call below
+ * forgets all decisions.  No counterpart in the reference.
+ */
+void cuttClearPlanCache(void);
+
+/*
  * After cuttPlanMeasure: the candidates of its most recent call in this
  * process, in enumeration order (a variant of the winner that beat it is
  * appended at the end).  usMeasured is 0 for candidates that were not timed

@@ -44,6 +44,7 @@ int main(void) {
   cuttSetMethodOverride(CUTT_METHOD_TILED);
   if (cuttGetMethodOverride() != CUTT_METHOD_TILED) return 26;
   cuttSetMethodOverride(0);
+  cuttClearPlanCache();
   printf("c abi ok, %d candidates, best method %d\n", n, info.method);
   return 0;
 }

@@ -367,3 +367,59 @@ def test_trivial_copy_sizes_alignments_and_cache_policies(gpu):
             del a, b
         assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
     assert policies == {0, 1, 3}
+
+
+def test_planning_the_same_tensor_again_reuses_the_decision(gpu, monkeypatch):
+    # cuttPlan keeps its last decisions: the second plan for a tensor is the same plan, made without
+    # the enumeration and the cost model; both plans own their tables (destroying one leaves the
+    # other working); another method override or CUTT_PLAN_CACHE=0 plans from scratch.
+    import torch
+    import cutt_amd as cutt
+    import oracle
+    dim, perm, es = (30, 3, 20, 9, 24, 29), (5, 2, 0, 4, 1, 3), 4
+    vol = int(np.prod(dim))
+    st = gpu.stream_handle()
+    data = gpu.seeded(vol, es, seed=11)
+    want = oracle.transpose_mt(list(dim), list(perm), data, 8)
+    d_in = gpu.to_device(data)
+    d_out = torch.full_like(d_in, -1)
+
+    def plan():
+        rc, h = cutt.cuttPlan(len(dim), dim, perm, es, st)
+        assert rc == cutt.CUTT_SUCCESS
+        d = cutt.get_plan_info(h).as_dict()
+        return h, d, d.pop("planMs")
+
+    def runs_right(h):
+        d_out.fill_(-1)
+        gpu.run_plan(h, d_in, d_out)
+        return np.array_equal(gpu.to_host(d_out, es), want)
+
+    cutt.clear_plan_cache()
+    h1, info1, ms1 = plan()
+    h2, info2, ms2 = plan()
+    say("plan ms: first %.3f, again %.3f (%s, %d candidates)" % (ms1, ms2, info1["method_name"], info1["numCandidates"]))
+    assert info1 == info2 and info1["method_name"] in ("Packed", "PackedSplit")
+    assert ms2 < 0.5 * ms1
+    assert cutt.cuttDestroy(h1) == cutt.CUTT_SUCCESS
+    assert runs_right(h2)
+    assert cutt.cuttDestroy(h2) == cutt.CUTT_SUCCESS
+
+    cutt.set_method_override(cutt.METHOD_TILED)
+    try:
+        h3, info3, _ = plan()
+        assert info3["method_name"] == "Tiled" and runs_right(h3)
+        assert cutt.cuttDestroy(h3) == cutt.CUTT_SUCCESS
+    finally:
+        cutt.set_method_override(0)
+
+    monkeypatch.setenv("CUTT_PLAN_CACHE", "0")
+    h4, info4, ms4 = plan()
+    assert info4 == info1 and ms4 > 2 * ms2 and runs_right(h4)
+    assert cutt.cuttDestroy(h4) == cutt.CUTT_SUCCESS
+    monkeypatch.delenv("CUTT_PLAN_CACHE")
+
+    cutt.clear_plan_cache()
+    h5, info5, ms5 = plan()
+    assert info5 == info1 and ms5 > 2 * ms2
+    assert cutt.cuttDestroy(h5) == cutt.CUTT_SUCCESS
