@@ -108,6 +108,8 @@ typedef struct cuttHipTiledArgs {
                          grid has 8*xcdChunk workgroups */
   uint32_t superM, superK;
   int cachePolicy;    /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
+  int grouped;        /* 0: a lane has all 16 rows of its tile in flight at once; 1: four at a time
+                         (each group of 16 tile rows is waited for before the next is requested) */
   cuttHipMbar mbar;
 } cuttHipTiledArgs;
 

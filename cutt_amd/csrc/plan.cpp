@@ -498,6 +498,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
+    a.grouped = opt.tiledGrouped > 0 ? 1 : 0;  // -1: decided from the model's estimate later
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
     plan.ldsBytes = (size_t)kTile * (kTile + 1) * pb.elemSize;
   } else {

@@ -70,8 +70,8 @@ bool benchTensor(const std::vector<int>& dimIn, const std::vector<int>& permIn) 
   if (usePlanTimer) std::printf("plan took %f ms\n", planMs);
   cuttPlanInfo info;
   CUTT_CHECK(cuttGetPlanInfo(plan, &info));
-  std::printf("method %s blocks %lld threads %d lds %llu candidates %d\n", methodNames[info.method], info.numBlocks,
-              info.numThreads, info.ldsBytes, info.numCandidates);
+  std::printf("method %s blocks %lld threads %d lds %llu candidates %d%s\n", methodNames[info.method], info.numBlocks,
+              info.numThreads, info.ldsBytes, info.numCandidates, info.tiledGrouped ? " rows-in-groups" : "");
   // what the cost model counted for this plan, to set beside hardware counters (128-byte lines)
   std::printf("model: predicted %.1f us, lines read %.0f written %.0f partly written %.0f, LDS cycles %.0f\n", info.usPredicted,
               info.rdLines, info.wrLines, info.wrPartialLines, info.ldsCycles);

@@ -54,6 +54,7 @@ typedef struct cuttPlanInfo {
   /* cost model: work items between the accesses to the two parts of a line shared by neighbouring
    * runs, on the read and on the write side (0 = no such neighbour) */
   double rdEdgeDist, wrEdgeDist;
+  int tiledGrouped;     /* Tiled: 1 if a lane keeps 4 instead of 16 tile rows in flight */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */

@@ -423,3 +423,28 @@ def test_planning_the_same_tensor_again_reuses_the_decision(gpu, monkeypatch):
     h5, info5, ms5 = plan()
     assert info5 == info1 and ms5 > 2 * ms2
     assert cutt.cuttDestroy(h5) == cutt.CUTT_SUCCESS
+
+
+def test_tiled_with_four_rows_per_lane_in_flight(gpu, monkeypatch):
+    # The Tiled kernel's second instance (a lane requests its 16 tile rows four at a time): forced
+    # on shapes with full, edge and thin tiles, both widths; then chosen by the planner itself on a
+    # large tensor of 4-byte elements whose rows start off the 128-byte grid.
+    import cutt_amd as cutt
+    cases = [((43, 67), (1, 0)), ((64, 64), (1, 0)), ((65, 127, 3), (1, 0, 2)), ((130, 9, 70), (2, 1, 0)),
+             ((1000, 30, 777), (2, 1, 0)), ((17, 5, 300), (2, 1, 0)), ((300, 5, 17), (2, 1, 0)),
+             ((129, 3, 257, 31), (2, 1, 0, 3))]
+    monkeypatch.setenv("CUTT_TILED_GROUPED", "1")
+    cutt.set_method_override(cutt.METHOD_TILED)
+    try:
+        for dim, perm in cases:
+            for es in (4, 8):
+                say("grouped tiled dim=%s perm=%s es=%d" % (dim, perm, es))
+                info = gpu.check_case(list(dim), list(perm), es)
+                assert info.method_name == "Tiled" and info.tiledGrouped == 1
+    finally:
+        cutt.set_method_override(0)
+    monkeypatch.delenv("CUTT_TILED_GROUPED")
+    for es, want in ((4, 1), (8, 0)):
+        say("planner's own choice, es=%d" % es)
+        info = gpu.check_case([4457, 44570], [1, 0], es)
+        assert info.method_name == "Tiled" and info.tiledGrouped == want

@@ -168,3 +168,18 @@ def test_plans_do_not_depend_on_the_number_of_planner_threads(cutt, monkeypatch)
             infos, best = method_set(cutt, dim, perm, es)
             got.append(([i.as_dict() for i in infos], best.as_dict()))
         assert got[0] == got[1] == got[2]
+
+
+def test_rows_in_groups_only_for_large_unaligned_tensors_of_4_byte_elements(cutt):
+    def tiled(dim, perm, es):
+        infos, best = method_set(cutt, dim, perm, es)
+        t = [i for i in infos if i.method_name == "Tiled"]
+        assert len(t) == 1
+        return t[0].tiledGrouped
+    assert tiled((4457, 44570), (1, 0), 4) == 1          # rows of 17828 bytes, 795 MB
+    assert tiled((1535, 157, 895), (2, 1, 0), 4) == 1
+    assert tiled((4457, 44570), (1, 0), 8) == 0          # 8-byte elements
+    assert tiled((8192, 8192), (1, 0), 4) == 0           # aligned rows
+    assert tiled((1536, 157, 896), (2, 1, 0), 4) == 0    # aligned rows
+    assert tiled((445, 4457), (1, 0), 4) == 0            # fits the memory-side cache
+    assert tiled((31, 97, 101, 659), (3, 1, 2, 0), 4) == 0   # thin tiles: 2 requested lines per line of data
