@@ -232,11 +232,16 @@ void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
   const double lines = bytes / 128.0;
   if (cache > 0 && bytes <= 3.5 * cache) {
     // ... unless the plan reads each line from several requests (more than ~1.7 lines requested
-    // per line of data): then the re-reads must find the line in the caches (0.85-0.97 x)
-    // (a Tiled plan's 256-byte rows of 4-byte elements share every third line with the
-    // neighbouring tile: from 1.5 lines per line of data on, ordinary loads measured 3 % faster)
+    // per line of data): then the re-reads must find the line in the caches (0.85-0.97 x).
+    // A Tiled plan's 256-byte rows of 4-byte elements share every third line with the neighbouring
+    // tile: there the limit is 1.5, except between 0.8 and 1.8 cache sizes per buffer, where it is
+    // 1.6 (at 1.56 lines per line of data: ordinary loads +10 % at 0.75 cache sizes and +7...+15 %
+    // at 2.1-3.1, streaming loads +9...+18 % at 0.88-1.56), and a plan that keeps four rows per
+    // lane in flight always streams its reads (+2...+24 % over ordinary loads at 1-3.4 cache sizes).
     const bool narrowTiles = (p.method == kTiled || p.method == kTiledCopy) && p.pb.elemSize == 4;
-    setCachePolicy(p, p.model.rdLines < (narrowTiles ? 1.5 : 1.7) * lines ? 1 : 0);
+    const double limit = narrowTiles ? (bytes >= 0.8 * cache && bytes < 1.8 * cache ? 1.6 : 1.5) : 1.7;
+    const bool grouped = p.method == kTiled && p.tiled.grouped;
+    setCachePolicy(p, grouped || p.model.rdLines < limit * lines ? 1 : 0);
     return;
   }
   const bool wholeReads = p.model.rdLines <= 1.15 * lines;
@@ -271,8 +276,8 @@ void parallelFor(int n, F&& f) {
 }
 
 // A Tiled plan on 4-byte elements whose tile rows start off the 128-byte grid (the model counts
-// 1.2-1.6 requested lines per line of data on both sides) and whose tensor is well beyond the
-// memory-side cache keeps four instead of sixteen rows per lane in flight.  Measured on 236 such
+// 1.2-1.6 requested lines per line of data on both sides) and whose tensor is larger than the
+// memory-side cache (from 1.1 cache sizes per buffer on) keeps four instead of sixteen rows per lane in flight.  Measured on 236 such
 // plans of the reference's random-tensor suites: median +4.7 %, mean +4.2 %, none more than 3.4 %
 // slower; outside these limits the same switch costs up to 14 % (aligned or cache-sized tensors,
 // 8-byte elements).  (Not applied when CUTT_TILED_GROUPED pins the switch.)
@@ -282,7 +287,7 @@ void chooseTiledGrouping(Plan& p, const cuttHipDeviceProps& props) {
   const double lines = bytes / 128.0;
   const double cache = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
   const double rdAmp = p.model.rdLines / lines, wrAmp = p.model.wrLines / lines;
-  const bool grouped = p.pb.elemSize == 4 && bytes > 1.5 * cache && rdAmp > 1.2 && rdAmp < 1.6 && wrAmp > 1.2 &&
+  const bool grouped = p.pb.elemSize == 4 && bytes > 1.1 * cache && rdAmp > 1.2 && rdAmp < 1.6 && wrAmp > 1.2 &&
                        wrAmp < 1.6;
   p.tiled.grouped = grouped ? 1 : 0;
   if (grouped) p.model.usPredicted *= 0.96;
