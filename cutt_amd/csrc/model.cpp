@@ -422,9 +422,14 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // measured 5-10 % between 4 KB and 64 KB of staged data.
     factor -= 0.10 * (double)plan.ldsBytes / 65536.0;
     // ... and for 4-byte elements most of that comes below 32 KB: over all candidates of 48 random
-    // tensors of ranks 4-7 that the model rated within 15 % of its best, items of less than 12 KB ran
-    // as predicted, those of 28 KB and more 6-7 % faster than predicted.
-    if (es == 4) factor -= 0.07 * std::min(1.0, (double)plan.ldsBytes / 32768.0);
+    // tensors of ranks 4-7 (0.4-0.9 GB) that the model rated within 15 % of its best, items of less
+    // than 12 KB ran as predicted, those of 28 KB and more 6-7 % faster than predicted.  Tensors that
+    // fit the memory-side cache are another matter (there the few large items of such a plan cost
+    // up to 30 %), so the term applies beyond one cache size per buffer only.
+    {
+      const double cache = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
+      if (es == 4 && bytes > cache) factor -= 0.07 * std::min(1.0, (double)plan.ldsBytes / 32768.0);
+    }
     // LDS bank conflicts of the gather, and table reloads when a block has few items.
     factor += 0.5 * r.ldsCycles / ((double)props.cuCount * props.clockKHz * 1e3) / tCopy;
     factor += 0.25 * tableBytes / (2.0 * bytes);
