@@ -250,18 +250,25 @@ void chooseCachePolicy(Plan& p, const cuttHipDeviceProps& props) {
 }
 
 // Runs f(0) .. f(n-1) on up to eight host threads (CUTT_PLAN_THREADS caps the number; 1 = the
-// calling thread only) and returns when all have finished.  The calls must not depend on each
-// other: the model's estimate of a candidate is a pure function of that candidate, so a plan does
-// not depend on the number of threads.
+// calling thread only) and returns when all have finished; false if a call threw (out of memory).
+// The calls must not depend on each other: the model's estimate of a candidate is a pure function
+// of that candidate, so a plan does not depend on the number of threads.
 template <class F>
-void parallelFor(int n, F&& f) {
+bool parallelFor(int n, F&& f) {
   int cap = 8;
   if (const char* e = std::getenv("CUTT_PLAN_THREADS")) cap = std::max(1, std::atoi(e));
   const unsigned hw = std::thread::hardware_concurrency();
   const int nt = std::min({n, cap, hw ? (int)hw : 1});
   std::atomic<int> next{0};
+  std::atomic<bool> threw{false};
   auto work = [&]() {
-    for (int i = next.fetch_add(1); i < n; i = next.fetch_add(1)) f(i);
+    for (int i = next.fetch_add(1); i < n; i = next.fetch_add(1)) {
+      try {
+        f(i);
+      } catch (...) {
+        threw = true;
+      }
+    }
   };
   std::vector<std::thread> helpers;
   for (int t = 1; t < nt; t++) {
@@ -273,14 +280,16 @@ void parallelFor(int n, F&& f) {
   }
   work();
   for (std::thread& t : helpers) t.join();
+  return !threw;
 }
 
 // A Tiled plan on 4-byte elements whose tile rows start off the 128-byte grid (the model counts
 // 1.2-1.6 requested lines per line of data on both sides) and whose tensor is larger than the
-// memory-side cache (from 1.1 cache sizes per buffer on) keeps four instead of sixteen rows per lane in flight.  Measured on 236 such
-// plans of the reference's random-tensor suites: median +4.7 %, mean +4.2 %, none more than 3.4 %
-// slower; outside these limits the same switch costs up to 14 % (aligned or cache-sized tensors,
-// 8-byte elements).  (Not applied when CUTT_TILED_GROUPED pins the switch.)
+// memory-side cache (from 1.1 cache sizes per buffer on) keeps four instead of sixteen rows per
+// lane in flight.  Measured on such plans of the reference's random-tensor suites: +5 % in the
+// median at 0.8 GB per buffer (164 plans, worst -3.5 %, best +17 %), single tensors +20...+34 % at
+// 0.3-0.5 GB; outside these limits the same switch costs up to 14 % (aligned or cache-sized
+// tensors, 8-byte elements).  (Not applied when CUTT_TILED_GROUPED pins the switch.)
 void chooseTiledGrouping(Plan& p, const cuttHipDeviceProps& props) {
   if (p.method != kTiled || std::getenv("CUTT_TILED_GROUPED")) return;
   const double bytes = (double)p.pb.volume * p.pb.elemSize;
@@ -303,10 +312,10 @@ bool estimateAndTune(Plan& p, const cuttHipDeviceProps& props) {
 // Model estimate of every candidate; false if one of them fails.
 bool estimateAll(std::vector<Plan>& plans, const cuttHipDeviceProps& props) {
   std::atomic<bool> ok{true};
-  parallelFor((int)plans.size(), [&](int i) {
+  const bool ran = parallelFor((int)plans.size(), [&](int i) {
     if (!estimateAndTune(plans[i], props)) ok = false;
   });
-  return ok;
+  return ran && ok;
 }
 
 PlannerOptions plannerOptions(int forceMethod);
@@ -332,7 +341,8 @@ void refineMbarOrder(std::vector<Plan>& plans, const cuttHipDeviceProps& props, 
   for (size_t k = 0; k < idx.size() && k < 3; k++)
     for (int order : {0, 1, 2})
       if (order != base.mbarOrder) trials.push_back({idx[k], order, false, Plan()});
-  parallelFor((int)trials.size(), [&](int i) {
+  // a trial that fails or throws keeps ok == false and is passed over
+  (void)parallelFor((int)trials.size(), [&](int i) {
     Trial& t = trials[i];
     PlannerOptions opt = base;
     opt.mbarOrder = t.order;
@@ -414,8 +424,8 @@ cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int device
 
 }  // namespace
 
-extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
-                               size_t sizeofType, hipStream_t stream) {
+static cuttResult planImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
+                           size_t sizeofType, hipStream_t stream) {
   const auto t0 = std::chrono::steady_clock::now();
   if (!handle) return CUTT_INVALID_PARAMETER;
   cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
@@ -448,8 +458,8 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
   return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
 }
 
-extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, int* permutation,
-                                      size_t sizeofType, hipStream_t stream, void* idata, void* odata) {
+static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                  size_t sizeofType, hipStream_t stream, void* idata, void* odata) {
   const auto t0 = std::chrono::steady_clock::now();
   if (!handle) return CUTT_INVALID_PARAMETER;
   cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
@@ -481,12 +491,17 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   if (const char* e = std::getenv("CUTT_MEASURE_ALL"))
     if (std::atoi(e) != 0) margin = 1e30;
 
-  void *evStart = nullptr, *evStop = nullptr;
-  if (cuttHipEventCreate(&evStart) != 0) return CUTT_INTERNAL_ERROR;
-  if (cuttHipEventCreate(&evStop) != 0) {
-    cuttHipEventDestroy(evStart);
-    return CUTT_INTERNAL_ERROR;
-  }
+  // the two events of the timed runs; destroyed on every way out of this function
+  struct Events {
+    void *start = nullptr, *stop = nullptr;
+    ~Events() {
+      if (start) cuttHipEventDestroy(start);
+      if (stop) cuttHipEventDestroy(stop);
+    }
+  } events;
+  if (cuttHipEventCreate(&events.start) != 0 || cuttHipEventCreate(&events.stop) != 0) return CUTT_INTERNAL_ERROR;
+  void* const evStart = events.start;
+  void* const evStop = events.stop;
   double bestUs = 1e300;
   bool failed = false;
   // Times plan p (two runs, the faster counts); returns false on a HIP error.
@@ -605,8 +620,6 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
       if (tryVariant(v, false)) cur = v;
     }
   }
-  cuttHipEventDestroy(evStart);
-  cuttHipEventDestroy(evStop);
   if (failed || best < 0) return CUTT_INTERNAL_ERROR;
 
   {
@@ -621,8 +634,8 @@ extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, in
   return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), bestUs, t0);
 }
 
-extern "C" cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* dim, int* permutation,
-                                            size_t sizeofType, hipStream_t stream, int index) {
+static cuttResult planFromCandidateImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                        size_t sizeofType, hipStream_t stream, int index) {
   const auto t0 = std::chrono::steady_clock::now();
   if (!handle) return CUTT_INVALID_PARAMETER;
   cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
@@ -640,6 +653,35 @@ extern "C" cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* d
   if (index < 0 || index >= (int)plans.size()) return CUTT_INVALID_PARAMETER;
   if (!estimateAndTune(plans[index], props)) return CUTT_INTERNAL_ERROR;
   return storePlan(handle, std::move(plans[index]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
+}
+
+// The C entry points that plan: nothing a planner throws (std::bad_alloc from its tables) may
+// cross the C boundary; the caller gets CUTT_INTERNAL_ERROR instead.
+extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
+                               size_t sizeofType, hipStream_t stream) {
+  try {
+    return planImpl(handle, rank, dim, permutation, sizeofType, stream);
+  } catch (...) {
+    return CUTT_INTERNAL_ERROR;
+  }
+}
+
+extern "C" cuttResult cuttPlanMeasure(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                      size_t sizeofType, hipStream_t stream, void* idata, void* odata) {
+  try {
+    return planMeasureImpl(handle, rank, dim, permutation, sizeofType, stream, idata, odata);
+  } catch (...) {
+    return CUTT_INTERNAL_ERROR;
+  }
+}
+
+extern "C" cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* dim, int* permutation,
+                                            size_t sizeofType, hipStream_t stream, int index) {
+  try {
+    return planFromCandidateImpl(handle, rank, dim, permutation, sizeofType, stream, index);
+  } catch (...) {
+    return CUTT_INTERNAL_ERROR;
+  }
 }
 
 extern "C" cuttResult cuttDestroy(cuttHandle handle) {
