@@ -411,11 +411,10 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // random tensors ran 1.29-1.37 times (median) as long as predicted; every other class of tile
     // counts stayed within 6 % of its prediction.
     if (!copy && es == 4 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.3;
-    // The same shape with 8-byte elements (output runs of 65..128 elements, up to three tiles along
-    // Mm): 9 such candidates among 160 random tensors of ranks 3-7 ran 1.04-1.52 times as long as
-    // predicted (mean 1.24, but half of them below 1.15, so the factor is a cautious one), the other
-    // tile counts within 10 % in the mean.
-    if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 3.0) factor *= 1.1;
+    // The same shape with 8-byte elements: 51 forced plans with two tiles along Mk and one or two
+    // along Mm ran 1.11 times as long as predicted in the mean (0.84-1.37), those with three and
+    // more tiles along Mm 0.97 times.
+    if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.1;
   } else {
     factor = 1.05 + (es == 4 ? 0.17 : 0.093) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
