@@ -404,7 +404,12 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double rdSlots = tilesM * kTile * rows16(volMk);
     const double wrSlots = copy ? rdSlots : rows16(volMm) * tilesK * kTile;
     const double waste = 0.5 * (rdSlots + wrSlots) / (volMm * volMk) - 1.0;
-    factor = (es == 4 ? 1.00 : 0.95) + 0.25 * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
+    // Slots of a tile that hold no element cost 4-byte elements half of what they cost 8-byte ones
+    // (280 forced plans with a single tile along Mm or Mk: with 0.25 the 4-byte ones ran 0.91 /
+    // 0.96 / 1.00 times the prediction at extents 17-32 / 33-48 / 49-64, the 8-byte ones 0.93-0.97
+    // whatever the extent; a constant 0.95 for those was tried and only moved single tensors by
+    // 25 % in both directions).
+    factor = (es == 4 ? 1.00 : 0.95) + (es == 4 ? 0.12 : 0.25) * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? (es == 4 ? 0.20 : 0.10) : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
     // Tiny slabs of 4-byte elements: with one or two tiles along Mm and exactly two along Mk (a
     // 65..128-long output run cut into a 256-byte piece and a remainder), 46 such plans among 3000
