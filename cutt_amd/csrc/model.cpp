@@ -409,7 +409,12 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // 0.96 / 1.00 times the prediction at extents 17-32 / 33-48 / 49-64, the 8-byte ones 0.93-0.97
     // whatever the extent; a constant 0.95 for those was tried and only moved single tensors by
     // 25 % in both directions).
-    factor = (es == 4 ? 1.00 : 0.95) + (es == 4 ? 0.12 : 0.25) * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
+    // (Measured on tensors of 0.4-0.9 GB; a tensor that fits the memory-side cache keeps 0.25: with
+    // 0.12 a 45 MB tensor with 30-wide tiles was planned Tiled at 58 % of memcpy instead of
+    // PackedSplit at 78 %.)
+    const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
+    const double wasteCost = es == 4 && bytes > cacheBytes ? 0.12 : 0.25;
+    factor = (es == 4 ? 1.00 : 0.95) + wasteCost * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
              (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? (es == 4 ? 0.20 : 0.10) : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
     // Tiny slabs of 4-byte elements: with one or two tiles along Mm and exactly two along Mk (a
     // 65..128-long output run cut into a 256-byte piece and a remainder), 46 such plans among 3000
@@ -419,7 +424,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // The same shape with 8-byte elements: 51 forced plans with two tiles along Mk and one or two
     // along Mm ran 1.11 times as long as predicted in the mean (0.84-1.37), those with three and
     // more tiles along Mm 0.97 times.
-    if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0) factor *= 1.1;
+    if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0 && bytes > cacheBytes) factor *= 1.1;  // measured at 1.9-3.7 GB
   } else {
     factor = 1.05 + (es == 4 ? 0.17 : 0.093) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
