@@ -183,3 +183,28 @@ def test_rows_in_groups_only_for_large_unaligned_tensors_of_4_byte_elements(cutt
     assert tiled((1536, 157, 896), (2, 1, 0), 4) == 0    # aligned rows
     assert tiled((445, 4457), (1, 0), 4) == 0            # fits the memory-side cache
     assert tiled((31, 97, 101, 659), (3, 1, 2, 0), 4) == 0   # thin tiles: 2 requested lines per line of data
+
+
+def test_random_shapes_every_candidate(cutt, oracle_mod):
+    # Seeded random problems of ranks 2-8 with extents that give several tiles, uneven slabs and
+    # fused ranks; every candidate of every problem is replayed on the CPU and compared with the
+    # oracle, with the device's LDS size and with 8 / 16 KB (which turns Packed plans into splits).
+    rng = np.random.default_rng(2024)
+    seen = set()
+    done = 0
+    while done < 250:
+        rank = int(rng.integers(2, 9))
+        dim = [int(d) for d in np.maximum(2, rng.integers(2, 200, size=rank) // rng.integers(1, 20, size=rank))]
+        vol = int(np.prod(dim))
+        if vol < 200 or vol > 150000:
+            continue
+        perm = [int(p) for p in rng.permutation(rank)]
+        if rng.random() < 0.3:  # ranks that stay adjacent and fuse
+            perm = sorted(perm[: rank // 2]) + perm[rank // 2:]
+        if perm == sorted(perm):
+            continue
+        es = 4 if rng.random() < 0.5 else 8
+        lds = int(rng.choice([0, 0, 8192, 16384]))
+        seen |= check_all_candidates(cutt, oracle_mod, dim, perm, es, lds=lds)
+        done += 1
+    assert {"Tiled", "TiledCopy", "Packed", "PackedSplit"} <= seen
