@@ -450,3 +450,36 @@ def test_tiled_with_four_rows_per_lane_in_flight(gpu, monkeypatch):
         say("planner's own choice, es=%d" % es)
         info = gpu.check_case([4457, 44570], [1, 0], es)
         assert info.method_name == "Tiled" and info.tiledGrouped == want
+
+
+def test_every_candidate_of_random_midsize_tensors(gpu):
+    # Seeded random tensors of 0.3-2 M elements, ranks 3-7: every candidate of the enumeration runs
+    # on the GPU (all elements-per-lane, cache-policy and offset-width instances the planner can
+    # produce at this size) and must give the oracle's bytes.
+    import cutt_amd as cutt
+    import oracle
+    rng = np.random.default_rng(77)
+    done, executed = 0, 0
+    methods = set()
+    while done < 40:
+        rank = int(rng.integers(3, 8))
+        f = rng.uniform(1, 10, size=rank)
+        vol = rng.uniform(3e5, 2e6)
+        dim = [int(d) for d in np.maximum(2, np.round(f * (vol / np.prod(f)) ** (1.0 / rank)))]
+        perm = [int(p) for p in rng.permutation(rank)]
+        if perm == sorted(perm):
+            continue
+        es = 4 if done % 2 else 8
+        v = int(np.prod(dim))
+        data = gpu.seeded(v, es, seed=done)
+        expect = oracle.transpose_mt(dim, perm, data, 8)
+        with cutt.Candidates(dim, perm, es) as c:
+            n = len(c)
+        say("random midsize %d: dim=%s perm=%s es=%d, %d candidates" % (done, dim, perm, es, n))
+        for i in range(n):
+            info = gpu.check_case(dim, perm, es, data=data, how="candidate", candidate=i, expect=expect)
+            methods.add(info.method_name)
+            executed += 1
+        done += 1
+    say("executed %d candidates" % executed)
+    assert {"Tiled", "Packed", "PackedSplit"} <= methods
