@@ -17,6 +17,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <list>
+#include <memory>
 #include <mutex>
 #include <string>
 #include <system_error>
@@ -41,7 +42,10 @@ struct StoredPlan {
 };
 
 std::mutex gMutex;
-std::unordered_map<cuttHandle, StoredPlan*> gPlans;
+// A handle maps to a shared owner: cuttExecute copies the pointer under the mutex and launches from
+// its copy, so a cuttDestroy of the same handle from another thread frees the plan (and its device
+// tables) only after that launch has been issued.
+std::unordered_map<cuttHandle, std::shared_ptr<StoredPlan>> gPlans;
 cuttHandle gNextHandle = 0;
 std::unordered_map<int, cuttHipDeviceProps> gDeviceProps;
 int gMethodOverride = -1;  // -1 = not initialised from the environment yet
@@ -151,6 +155,7 @@ bool currentDevice(int& deviceID, cuttHipDeviceProps& props) {
   if (it == gDeviceProps.end()) {
     cuttHipDeviceProps p;
     if (cuttHipGetDeviceProps(deviceID, &p) != 0) return false;
+    sanitizeDeviceProps(p);
     it = gDeviceProps.emplace(deviceID, p).first;
   }
   props = it->second;
@@ -401,24 +406,18 @@ bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
 
 cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int deviceID, int numCandidates,
                      double usMeasured, std::chrono::steady_clock::time_point t0) {
-  StoredPlan* sp = new StoredPlan();
+  std::shared_ptr<StoredPlan> sp = std::make_shared<StoredPlan>();
   sp->plan = std::move(chosen);
   sp->plan.stream = stream;
   sp->plan.deviceID = deviceID;
   sp->numCandidates = numCandidates;
   sp->usMeasured = usMeasured;
-  if (sp->plan.activate() != 0) {
-    delete sp;
-    return CUTT_INTERNAL_ERROR;
-  }
+  if (sp->plan.activate() != 0) return CUTT_INTERNAL_ERROR;
   sp->planMs = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
   std::lock_guard<std::mutex> lock(gMutex);
   *handle = gNextHandle++;
-  if (gPlans.count(*handle)) {
-    delete sp;
-    return CUTT_INTERNAL_ERROR;
-  }
-  gPlans.emplace(*handle, sp);
+  if (gPlans.count(*handle)) return CUTT_INTERNAL_ERROR;
+  gPlans.emplace(*handle, std::move(sp));
   return CUTT_SUCCESS;
 }
 
@@ -685,20 +684,20 @@ extern "C" cuttResult cuttPlanFromCandidate(cuttHandle* handle, int rank, int* d
 }
 
 extern "C" cuttResult cuttDestroy(cuttHandle handle) {
-  StoredPlan* sp = nullptr;
+  std::shared_ptr<StoredPlan> sp;
   {
     std::lock_guard<std::mutex> lock(gMutex);
     auto it = gPlans.find(handle);
     if (it == gPlans.end()) return CUTT_INVALID_PLAN;
-    sp = it->second;
+    sp = std::move(it->second);
     gPlans.erase(it);
   }
-  delete sp;
+  sp.reset();  // frees the plan outside the lock, unless a cuttExecute still holds it
   return CUTT_SUCCESS;
 }
 
 extern "C" cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata) {
-  StoredPlan* sp = nullptr;
+  std::shared_ptr<StoredPlan> sp;
   {
     std::lock_guard<std::mutex> lock(gMutex);
     auto it = gPlans.find(handle);

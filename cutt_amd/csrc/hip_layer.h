@@ -216,7 +216,14 @@ int cuttHipEventSynchronize(void* event);
 int cuttHipEventElapsedMs(void* start, void* stop, float* ms);
 const char* cuttHipErrorString(int err);
 
-/* ---- kernel launches (asynchronous on `stream`) -------------------------- */
+/* ---- kernel launches (asynchronous on `stream`) --------------------------
+ * A plan's arguments are checked once, when the plan is activated (cuttHipValidate*: shapes, grid,
+ * division constants, table pointers; 0 or a hipError_t value); the launch functions then only
+ * compute the grid and launch, and return the launch call's own result.  Launching arguments that
+ * did not pass their check is undefined. */
+int cuttHipValidateTiled(const cuttHipTiledArgs* args);
+int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* args);
+int cuttHipValidatePacked(const cuttHipPackedArgs* args);
 int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);

@@ -1,6 +1,7 @@
 /*
  * hip_layer.hip - HIP runtime side of the C-ABI layer declared in hip_layer.h:
- * device queries, allocation, copies, memset, events.  No device code here.
+ * device queries, allocation, copies, memset, events.  No device code here (the layer's plain
+ * arithmetic is in layer_math.cpp).
  *
  * Unlike the reference's helpers (reference src/CudaUtils.h:35-42 prints and
  * calls exit(1) on any runtime error) every function reports the error code
@@ -11,43 +12,6 @@
 #include <cstring>
 
 #include "hip_layer.h"
-
-extern "C" cuttHipDivisor cuttHipMakeDivisor(uint32_t d) {
-  cuttHipDivisor dv = {0u, 0u, 1u};  // d <= 1: n / 1
-  if (d >= 2) {
-    uint32_t shift = 0;
-    while ((1ull << (shift + 1)) < d) shift++;  // ceil(log2 d) - 1
-    const uint64_t pow2 = 1ull << (32 + shift);
-    dv.mul = (uint32_t)((pow2 + d - 1) / d);
-    dv.shift = shift;
-    dv.add = 0;
-  }
-  return dv;
-}
-
-extern "C" uint32_t cuttHipDivide(uint32_t n, cuttHipDivisor dv) {
-  const uint32_t hi = (uint32_t)(((uint64_t)n * dv.mul) >> 32);
-  return (hi + n * dv.add) >> dv.shift;
-}
-
-extern "C" int cuttHipFinishMbar(cuttHipMbar* mb) {
-  if (!mb || mb->n < 0 || mb->n > CUTT_MAX_RANK) return -1;
-  uint64_t below = 1;
-  for (int k = 0; k < CUTT_MAX_RANK; k++) {
-    cuttHipMbarDim& d = mb->d[k];
-    if (k >= mb->n) {
-      d.belowMul = d.extentMul = d.ctl = 0;  // quotients 0: no contribution
-      continue;
-    }
-    if (d.extent == 0 || below * d.extent >= (1ull << 31)) return -1;
-    const cuttHipDivisor b = cuttHipMakeDivisor((uint32_t)below), e = cuttHipMakeDivisor(d.extent);
-    d.belowMul = b.mul;
-    d.extentMul = e.mul;
-    d.ctl = b.shift | (e.shift << 8) | (b.add << 16) | (e.add << 17);
-    below *= d.extent;
-  }
-  return 0;
-}
 
 extern "C" int cuttHipGetDevice(int* device) { return (int)hipGetDevice(device); }
 

@@ -34,6 +34,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <tuple>
+#include <type_traits>
 
 #include "hip_layer.h"
 #include "mbar_decode.h"
@@ -447,11 +449,6 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   }
 }
 
-size_t packedLdsBytes(const cuttHipPackedArgs* a) {
-  const size_t b = (size_t)a->ldsElems * a->elemSize;
-  return (b + 15) & ~(size_t)15;
-}
-
 // The table must carry the division constants cuttHipFinishMbar derives from its extents.
 bool mbarOk(const cuttHipMbar& mb) {
   cuttHipMbar want = mb;
@@ -515,19 +512,6 @@ __global__ __launch_bounds__(kCopyThreads) void copyKernel(const Vec16* __restri
 
 }  // namespace
 
-extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) { return packedLdsBytes(a); }
-
-// Registers per lane of packedKernel<T, E, *, WIDE> as compiled for gfx950 (the cache policy does
-// not change the count).  Rows: E = 1, 2, 4, 8, 16.
-extern "C" int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets) {
-  static const int narrow4[5] = {15, 23, 39, 68, 124}, wide4[5] = {18, 25, 40, 72, 128};
-  static const int narrow8[5] = {16, 25, 42, 80, 0}, wide8[5] = {18, 28, 48, 88, 0};
-  int row = 0;
-  while (row < 5 && (1 << row) != elemsPerThread) row++;
-  if (row == 5 || (elemSize != 4 && elemSize != 8)) return 0;
-  return elemSize == 4 ? (wideOffsets ? wide4 : narrow4)[row] : (wideOffsets ? wide8 : narrow8)[row];
-}
-
 extern "C" int cuttHipPackedRegsPerLaneLoaded(int elemSize, int elemsPerThread, int wideOffsets) {
   const void* f = nullptr;
 #define CUTT_PICK(T, E)                                                                       \
@@ -559,8 +543,25 @@ extern "C" int cuttHipPackedRegsPerLaneLoaded(int elemSize, int elemsPerThread, 
   return attr.numRegs;
 }
 
-extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, void* out, void* stream) {
-  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+namespace {
+
+// A launch reports the launch call's own result.  (hipGetLastError after a launch would also report
+// - and clear - an error that an earlier, unrelated call of the application left behind on this
+// thread, such as hipErrorNotReady from a stream query.)
+template <typename... KArgs, typename... Args>
+hipError_t launchKernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args... args) {
+  static_assert(sizeof...(KArgs) == sizeof...(Args), "one argument per kernel parameter");
+  std::tuple<std::remove_const_t<KArgs>...> held{args...};
+  void* ptrs[sizeof...(KArgs)];
+  int i = 0;
+  std::apply([&](auto&... v) { ((ptrs[i++] = (void*)&v), ...); }, held);
+  return hipLaunchKernel(reinterpret_cast<const void*>(kernel), grid, block, ptrs, lds, s);
+}
+
+}  // namespace
+
+extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
+  if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
       a->order < 0 || a->order > 5 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1))
@@ -569,18 +570,24 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
+  return 0;
+}
+
+extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, void* out, void* stream) {
+  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+  uint64_t blocks = 0;
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+    return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);
-#define CUTT_LAUNCH_TILED(T, NT)                                                                         \
-  if (a->grouped)                                                                                       \
-    hipLaunchKernelGGL((tiledKernel<T, NT, true>), grid, block, 0, s, *a, (const T*)in, (T*)out);       \
-  else                                                                                                  \
-    hipLaunchKernelGGL((tiledKernel<T, NT, false>), grid, block, 0, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_TILED(T, NT)                                                                        \
+  return (int)(a->grouped ? launchKernel(tiledKernel<T, NT, true>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
+                          : launchKernel(tiledKernel<T, NT, false>, grid, block, 0, s, *a, (const T*)in, (T*)out))
 #define CUTT_LAUNCH_TILED_NT(T)                                \
   switch (a->cachePolicy) {                                    \
-    case 0: CUTT_LAUNCH_TILED(T, 0); break;                    \
-    case 1: CUTT_LAUNCH_TILED(T, 1); break;                    \
-    default: CUTT_LAUNCH_TILED(T, 3); break;                   \
+    case 0: CUTT_LAUNCH_TILED(T, 0);                           \
+    case 1: CUTT_LAUNCH_TILED(T, 1);                           \
+    default: CUTT_LAUNCH_TILED(T, 3);                          \
   }
   if (a->elemSize == 4) {
     CUTT_LAUNCH_TILED_NT(uint32_t)
@@ -589,12 +596,10 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   }
 #undef CUTT_LAUNCH_TILED_NT
 #undef CUTT_LAUNCH_TILED
-  return (int)hipGetLastError();
 }
 
-extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void* in, void* out,
-                                      void* stream) {
-  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+extern "C" int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* a) {
+  if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
       a->order < 0 || a->order > 5 || !mbarOk(a->mbar))
@@ -603,15 +608,24 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
+  return 0;
+}
+
+extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void* in, void* out,
+                                      void* stream) {
+  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+  uint64_t blocks = 0;
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+    return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);
 #define CUTT_LAUNCH_TCOPY(T, NT) \
-  hipLaunchKernelGGL((tiledCopyKernel<T, NT>), grid, block, 0, s, *a, (const T*)in, (T*)out)
+  return (int)launchKernel(tiledCopyKernel<T, NT>, grid, block, 0, s, *a, (const T*)in, (T*)out)
 #define CUTT_LAUNCH_TCOPY_NT(T)                                \
   switch (a->cachePolicy) {                                    \
-    case 0: CUTT_LAUNCH_TCOPY(T, 0); break;                    \
-    case 1: CUTT_LAUNCH_TCOPY(T, 1); break;                    \
-    default: CUTT_LAUNCH_TCOPY(T, 3); break;                   \
+    case 0: CUTT_LAUNCH_TCOPY(T, 0);                           \
+    case 1: CUTT_LAUNCH_TCOPY(T, 1);                           \
+    default: CUTT_LAUNCH_TCOPY(T, 3);                          \
   }
   if (a->elemSize == 4) {
     CUTT_LAUNCH_TCOPY_NT(uint32_t)
@@ -620,7 +634,6 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
   }
 #undef CUTT_LAUNCH_TCOPY_NT
 #undef CUTT_LAUNCH_TCOPY
-  return (int)hipGetLastError();
 }
 
 // Plain copy for the Trivial method.  Both pointers 16-byte aligned: copyKernel; otherwise the
@@ -637,16 +650,14 @@ extern "C" int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int ca
   if (blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
   const dim3 grid((uint32_t)blocks), block(kCopyThreads);
   switch (cachePolicy) {
-    case 0: hipLaunchKernelGGL(copyKernel<0>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords); break;
-    case 1: hipLaunchKernelGGL(copyKernel<1>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords); break;
-    default: hipLaunchKernelGGL(copyKernel<3>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords); break;
+    case 0: return (int)launchKernel(copyKernel<0>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
+    case 1: return (int)launchKernel(copyKernel<1>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
+    default: return (int)launchKernel(copyKernel<3>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
   }
-  return (int)hipGetLastError();
 }
 
 // Lets the packed kernels use more than the default 64 KB of dynamic LDS on the current device.
-// Called when a packed plan is activated (so that a plan's first cuttExecute already is a plain
-// kernel launch) and, as a cheap check, before every launch.
+// Called when a packed plan is activated, so that every cuttExecute is a plain kernel launch.
 extern "C" int cuttHipPreparePacked(void) {
   // Function attributes are kept per device.  Two threads may both find the flag clear and both
   // make the calls: they are idempotent.
@@ -676,8 +687,23 @@ extern "C" int cuttHipPreparePacked(void) {
   return 0;
 }
 
-extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, void* out, void* stream) {
-  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+// Number of workgroups of a packed launch (0 = the work items do not fit a grid).
+static uint64_t packedGrid(const cuttHipPackedArgs* a) {
+  uint64_t items = (uint64_t)a->volMbar;
+  for (int i = 0; i < 2; i++) {
+    items *= (uint64_t)std::max(1, a->split[i].numSplit);
+    if (items > 0x7fffffffull) return 0;
+  }
+  uint64_t blocks = (items + a->itemsPerBlock - 1) / a->itemsPerBlock;
+  if (a->xcdChunk) {
+    if ((uint64_t)a->xcdChunk * kNumXcd < blocks) return 0;
+    blocks = (uint64_t)a->xcdChunk * kNumXcd;
+  }
+  return blocks <= 0x7fffffffull ? blocks : 0;
+}
+
+extern "C" int cuttHipValidatePacked(const cuttHipPackedArgs* a) {
+  if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
       (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
       (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
@@ -688,14 +714,11 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
       // 32-bit byte offsets reach 4 GB
       (!a->wideOffsets && (uint64_t)a->volume * (uint64_t)a->elemSize > (1ull << 32)))
     return (int)hipErrorInvalidValue;
-  uint64_t items = (uint64_t)a->volMbar;
   for (int i = 0; i < 2; i++) {
     const cuttHipSplitRank& sr = a->split[i];
     if (sr.numSplit < 1 || sr.slabRem < 0 || sr.slabRem >= sr.numSplit || sr.slabFloor < 0 ||
         !divisorOk(sr.div, (uint32_t)sr.numSplit))
       return (int)hipErrorInvalidValue;
-    items *= (uint64_t)sr.numSplit;
-    if (items > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
   }
   for (int c = 0; c < 4; c++) {
     // class c is used only if the split ranks it refers to have slabs of the larger size
@@ -708,36 +731,33 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
     const uint32_t last = (uint32_t)k.vol - 1;
     if ((int)(last + (last >> a->padShift)) >= a->ldsElems) return (int)hipErrorInvalidValue;
   }
-  uint64_t blocks = (items + a->itemsPerBlock - 1) / a->itemsPerBlock;
-  if (blocks == 0) return (int)hipErrorInvalidConfiguration;
-  if (a->xcdChunk) {
-    if ((uint64_t)a->xcdChunk * kNumXcd < blocks) return (int)hipErrorInvalidValue;
-    blocks = (uint64_t)a->xcdChunk * kNumXcd;
-    if (blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
-  }
-  const size_t lds = packedLdsBytes(a);
+  if (packedGrid(a) == 0) return (int)hipErrorInvalidConfiguration;
+  return 0;
+}
 
-  if (int r = cuttHipPreparePacked(); r != 0) return r;
+extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, void* out, void* stream) {
+  if (!a || !in || !out) return (int)hipErrorInvalidValue;
+  const uint64_t blocks = packedGrid(a);
+  if (blocks == 0) return (int)hipErrorInvalidConfiguration;
+  const size_t lds = cuttHipPackedLdsBytes(a);
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(a->numThreads);
   const bool wide = a->wideOffsets != 0;
-#define CUTT_LAUNCH_PACKED(T, E, NT)                                                                    \
-  if (wide)                                                                                            \
-    hipLaunchKernelGGL((packedKernel<T, E, NT, true>), grid, block, lds, s, *a, (const T*)in, (T*)out); \
-  else                                                                                                 \
-    hipLaunchKernelGGL((packedKernel<T, E, NT, false>), grid, block, lds, s, *a, (const T*)in, (T*)out)
+#define CUTT_LAUNCH_PACKED(T, E, NT)                                                                              \
+  return (int)(wide ? launchKernel(packedKernel<T, E, NT, true>, grid, block, lds, s, *a, (const T*)in, (T*)out)  \
+                    : launchKernel(packedKernel<T, E, NT, false>, grid, block, lds, s, *a, (const T*)in, (T*)out))
 #define CUTT_LAUNCH_PACKED_NT(T, E)                            \
   switch (a->cachePolicy) {                                    \
-    case 0: CUTT_LAUNCH_PACKED(T, E, 0); break;                \
-    case 1: CUTT_LAUNCH_PACKED(T, E, 1); break;                \
-    default: CUTT_LAUNCH_PACKED(T, E, 3); break;               \
+    case 0: CUTT_LAUNCH_PACKED(T, E, 0);                       \
+    case 1: CUTT_LAUNCH_PACKED(T, E, 1);                       \
+    default: CUTT_LAUNCH_PACKED(T, E, 3);                      \
   }
 #define CUTT_LAUNCH_PACKED_E(T)                                \
   switch (a->elemsPerThread) {                                 \
-    case 1: CUTT_LAUNCH_PACKED_NT(T, 1) break;                 \
-    case 2: CUTT_LAUNCH_PACKED_NT(T, 2) break;                 \
-    case 4: CUTT_LAUNCH_PACKED_NT(T, 4) break;                 \
-    default: CUTT_LAUNCH_PACKED_NT(T, 8) break;                \
+    case 1: CUTT_LAUNCH_PACKED_NT(T, 1)                        \
+    case 2: CUTT_LAUNCH_PACKED_NT(T, 2)                        \
+    case 4: CUTT_LAUNCH_PACKED_NT(T, 4)                        \
+    default: CUTT_LAUNCH_PACKED_NT(T, 8)                       \
   }
   if (a->elemSize == 4 && a->elemsPerThread == 16) {
     // 4-byte elements only: 16 per lane stage the same 64 KB as 8 per lane do for 8-byte elements
@@ -750,5 +770,4 @@ extern "C" int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void* in, v
 #undef CUTT_LAUNCH_PACKED_NT
 #undef CUTT_LAUNCH_PACKED_E
 #undef CUTT_LAUNCH_PACKED
-  return (int)hipGetLastError();
 }

@@ -1,0 +1,60 @@
+/*
+ * layer_math.cpp - the part of the C-ABI layer (hip_layer.h) that is plain arithmetic: division
+ * constants, the Mbar table's derived fields, LDS bytes and register counts of the packed kernel.
+ * No HIP header and no runtime call, so the host planner can be linked and tested without the
+ * device side (the kernels check their arguments with the same functions).
+ */
+#include "hip_layer.h"
+
+extern "C" cuttHipDivisor cuttHipMakeDivisor(uint32_t d) {
+  cuttHipDivisor dv = {0u, 0u, 1u};  // d <= 1: n / 1
+  if (d >= 2) {
+    uint32_t shift = 0;
+    while ((1ull << (shift + 1)) < d) shift++;  // ceil(log2 d) - 1
+    const uint64_t pow2 = 1ull << (32 + shift);
+    dv.mul = (uint32_t)((pow2 + d - 1) / d);
+    dv.shift = shift;
+    dv.add = 0;
+  }
+  return dv;
+}
+
+extern "C" uint32_t cuttHipDivide(uint32_t n, cuttHipDivisor dv) {
+  const uint32_t hi = (uint32_t)(((uint64_t)n * dv.mul) >> 32);
+  return (hi + n * dv.add) >> dv.shift;
+}
+
+extern "C" int cuttHipFinishMbar(cuttHipMbar* mb) {
+  if (!mb || mb->n < 0 || mb->n > CUTT_MAX_RANK) return -1;
+  uint64_t below = 1;
+  for (int k = 0; k < CUTT_MAX_RANK; k++) {
+    cuttHipMbarDim& d = mb->d[k];
+    if (k >= mb->n) {
+      d.belowMul = d.extentMul = d.ctl = 0;  // quotients 0: no contribution
+      continue;
+    }
+    if (d.extent == 0 || below * d.extent >= (1ull << 31)) return -1;
+    const cuttHipDivisor b = cuttHipMakeDivisor((uint32_t)below), e = cuttHipMakeDivisor(d.extent);
+    d.belowMul = b.mul;
+    d.extentMul = e.mul;
+    d.ctl = b.shift | (e.shift << 8) | (b.add << 16) | (e.add << 17);
+    below *= d.extent;
+  }
+  return 0;
+}
+
+extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) {
+  const size_t b = (size_t)a->ldsElems * a->elemSize;
+  return (b + 15) & ~(size_t)15;
+}
+
+// Registers per lane of packedKernel<T, E, *, WIDE> as compiled for gfx950 (the cache policy does
+// not change the count).  Rows: E = 1, 2, 4, 8, 16.
+extern "C" int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets) {
+  static const int narrow4[5] = {15, 23, 39, 68, 124}, wide4[5] = {18, 25, 40, 72, 128};
+  static const int narrow8[5] = {16, 25, 42, 80, 0}, wide8[5] = {18, 28, 48, 88, 0};
+  int row = 0;
+  while (row < 5 && (1 << row) != elemsPerThread) row++;
+  if (row == 5 || (elemSize != 4 && elemSize != 8)) return 0;
+  return elemSize == 4 ? (wideOffsets ? wide4 : narrow4)[row] : (wideOffsets ? wide8 : narrow8)[row];
+}

@@ -58,6 +58,26 @@ cuttHipDeviceProps defaultMI355XProps() {
   return p;
 }
 
+// Runtimes and devices differ in what they report; a zero or implausible field would turn the
+// model's copy time into infinity (every candidate then ties) or size the grids for no CUs at all.
+void sanitizeDeviceProps(cuttHipDeviceProps& p) {
+  const cuttHipDeviceProps d = defaultMI355XProps();
+  if (p.cuCount < 1 || p.cuCount > 4096) p.cuCount = d.cuCount;
+  if (p.waveSize != 32 && p.waveSize != 64) p.waveSize = d.waveSize;
+  if (p.maxThreadsPerBlock < 64 || p.maxThreadsPerBlock > 1024) p.maxThreadsPerBlock = d.maxThreadsPerBlock;
+  if (p.maxThreadsPerCU < p.maxThreadsPerBlock) p.maxThreadsPerCU = d.maxThreadsPerCU;
+  if (p.ldsPerBlock < 16 * 1024) p.ldsPerBlock = std::min<size_t>(d.ldsPerBlock, 64 * 1024);
+  if (p.ldsPerCU < p.ldsPerBlock) p.ldsPerCU = p.ldsPerBlock;
+  if (p.clockKHz < 100000) p.clockKHz = d.clockKHz;
+  // the product of memory clock and bus width is what the model uses (bytes per second)
+  if (p.memClockKHz < 100000 || p.memBusWidthBits < 64) {
+    p.memClockKHz = d.memClockKHz;
+    p.memBusWidthBits = d.memBusWidthBits;
+  }
+  if (p.l2Bytes < 256 * 1024) p.l2Bytes = d.l2Bytes;
+  if (p.maxGridX < 65535) p.maxGridX = d.maxGridX;
+}
+
 // ---------------------------------------------------------------------------
 void Problem::set(int rank_, const int* dim_, const int* perm_, int elemSize_) {
   rank = rank_;
@@ -197,6 +217,8 @@ Plan& Plan::operator=(Plan&& o) noexcept {
   tablesBuilt = o.tablesBuilt;
   dTables = o.dTables;
   o.dTables = nullptr;
+  launchable = o.launchable;
+  o.launchable = false;
   model = o.model;
   return *this;
 }
@@ -227,6 +249,7 @@ Plan Plan::clone() const {
 }
 
 void Plan::release() {
+  if (method == kPacked || method == kPackedSplit) launchable = false;
   if (dTables) {
     cuttHipFree(dTables);
     dTables = nullptr;
@@ -825,7 +848,12 @@ bool Plan::buildTables() {
 }
 
 int Plan::activate() {
-  if (method != kPacked && method != kPackedSplit) return 0;
+  if (method == kTiled) return launchable ? 0 : ((launchable = cuttHipValidateTiled(&tiled) == 0) ? 0 : -1);
+  if (method == kTiledCopy) return launchable ? 0 : ((launchable = cuttHipValidateTiledCopy(&tcopy) == 0) ? 0 : -1);
+  if (method != kPacked && method != kPackedSplit) {
+    launchable = method == kTrivial;
+    return launchable ? 0 : -1;
+  }
   if (dTables) return 0;
   if (!buildTables()) return -1;
   if (int e = cuttHipPreparePacked(); e != 0) return e;
@@ -862,10 +890,16 @@ int Plan::activate() {
     packed.cls[c].rowOut = (const uint32_t*)(base + off[c][1]);
     packed.cls[c].shIdx = (const uint16_t*)(base + off[c][2]);
   }
+  if (int v = cuttHipValidatePacked(&packed); v != 0) {
+    release();
+    return v;
+  }
+  launchable = true;
   return 0;
 }
 
 int Plan::launch(const void* in, void* out) {
+  if (!launchable) return -1;  // activate() checks the arguments once; launches do not repeat that
   switch (method) {
     case kTrivial:
       return cuttHipLaunchCopy(in, out, (size_t)pb.volume * pb.elemSize, packed.cachePolicy, stream);

@@ -108,6 +108,7 @@ struct Plan {
   PackedTables tab[4];
   bool tablesBuilt = false;
   void* dTables = nullptr;
+  bool launchable = false;  // set by activate(): the launch arguments passed their check
 
   ModelResult model;
 
@@ -120,7 +121,7 @@ struct Plan {
 
   Plan clone() const;             // host-side copy of a plan that has no device tables yet
   bool buildTables();             // Packed/PackedSplit: fill tab[]; others: no-op
-  int activate();                 // upload tables; returns 0 or a HIP error code
+  int activate();                 // upload tables, check the launch arguments; 0 or an error code
   int launch(const void* in, void* out);  // asynchronous on stream
   void release();                 // free device tables
   std::string describe() const;
@@ -152,6 +153,8 @@ bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const Planner
 
 // Default device description of one MI355X, used when no GPU is present (tests, offline planning).
 cuttHipDeviceProps defaultMI355XProps();
+// Replace fields the runtime left at zero (or at implausible values) by those of the default.
+void sanitizeDeviceProps(cuttHipDeviceProps& props);
 
 }  // namespace cutt
 

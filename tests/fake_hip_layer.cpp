@@ -1,0 +1,63 @@
+// A stand-in for the runtime half of the library's internal C-ABI layer (cutt_amd/csrc/hip_layer.h),
+// for host-only tests of the plan API: "device" memory is host memory, a "launch" reads every word
+// of the plan's index tables (so that a sanitizer sees a plan freed under a running cuttExecute)
+// and takes a little time, events and synchronisation do nothing.  The layer's arithmetic
+// (division constants, Mbar tables) is the library's own layer_math.cpp.
+// CUTT_FAKE_ZERO_PROPS=1 reports a device whose clock, bus width, CU count and L2 size read zero.
+#include <atomic>
+#include <chrono>
+#include <cstdlib>
+#include <cstring>
+#include <thread>
+
+#include "hip_layer.h"
+
+namespace cutt {
+cuttHipDeviceProps defaultMI355XProps();
+}
+
+static std::atomic<uint64_t> gSink;
+
+static void touch(const cuttHipPackedArgs* a) {
+  uint64_t sum = 0;
+  for (int c = 0; c < 4; c++) {
+    if (((c & 1) && a->split[0].slabRem == 0) || ((c & 2) && a->split[1].slabRem == 0)) continue;
+    const cuttHipPackedClass& k = a->cls[c];
+    for (int i = 0; i < k.vol / k.inCont; i++) sum += k.rowIn[i];
+    for (int i = 0; i < k.vol / k.outCont; i++) sum += k.rowOut[i];
+    for (int i = 0; i < k.vol; i++) sum += k.shIdx[i];
+  }
+  gSink = sum;
+  std::this_thread::sleep_for(std::chrono::microseconds(50));
+}
+
+extern "C" {
+int cuttHipGetDevice(int* device) { *device = 0; return 0; }
+int cuttHipGetDeviceProps(int, cuttHipDeviceProps* p) {
+  *p = cutt::defaultMI355XProps();
+  const char* z = std::getenv("CUTT_FAKE_ZERO_PROPS");
+  if (z && std::atoi(z)) p->memClockKHz = p->memBusWidthBits = p->cuCount = p->l2Bytes = p->clockKHz = 0;
+  return 0;
+}
+int cuttHipMalloc(void** ptr, size_t bytes) { *ptr = std::malloc(bytes ? bytes : 1); return *ptr ? 0 : 2; }
+int cuttHipFree(void* ptr) { std::free(ptr); return 0; }
+int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes) { std::memcpy(dst, src, bytes); return 0; }
+int cuttHipMemcpyDtoDAsync(void* dst, const void* src, size_t bytes, void*) { std::memcpy(dst, src, bytes); return 0; }
+int cuttHipMemsetAsync(void* dst, int value, size_t bytes, void*) { std::memset(dst, value, bytes); return 0; }
+int cuttHipDeviceSynchronize(void) { return 0; }
+int cuttHipEventCreate(void** event) { *event = std::malloc(1); return 0; }
+int cuttHipEventDestroy(void* event) { std::free(event); return 0; }
+int cuttHipEventRecord(void*, void*) { return 0; }
+int cuttHipEventSynchronize(void*) { return 0; }
+int cuttHipEventElapsedMs(void*, void*, float* ms) { *ms = 1.0f; return 0; }
+const char* cuttHipErrorString(int) { return "fake layer"; }
+int cuttHipValidateTiled(const cuttHipTiledArgs* a) { return a ? 0 : 1; }
+int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* a) { return a ? 0 : 1; }
+int cuttHipValidatePacked(const cuttHipPackedArgs* a) { return a ? 0 : 1; }
+int cuttHipLaunchTiled(const cuttHipTiledArgs*, const void*, void*, void*) { return 0; }
+int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs*, const void*, void*, void*) { return 0; }
+int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void*, void*, void*) { touch(a); return 0; }
+int cuttHipLaunchCopy(const void*, void*, size_t, int, void*) { return 0; }
+int cuttHipPreparePacked(void) { return 0; }
+int cuttHipPackedRegsPerLaneLoaded(int, int, int) { return -1; }
+}
