@@ -10,7 +10,7 @@ from .api import (  # noqa: F401
     CUTT_INTERNAL_ERROR, CUTT_UNDEFINED_ERROR,
     METHOD_NAMES, METHOD_TRIVIAL, METHOD_PACKED, METHOD_PACKEDSPLIT, METHOD_TILED, METHOD_TILEDCOPY,
     CuttError, PlanInfo, lib, lib_path,
-    cuttPlan, cuttPlanMeasure, cuttPlanFromCandidate, cuttExecute, cuttDestroy,
+    cuttPlan, cuttPlanMeasure, cuttPlanFromCandidate, cuttExecute, cuttExecuteNoAlloc, cuttDestroy,
     get_plan_info, set_method_override, clear_plan_cache, get_last_measurement, reduce_ranks, Candidates,
 )
 from .build import build  # noqa: F401

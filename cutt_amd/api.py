@@ -93,6 +93,8 @@ def lib():
     l.cuttPlanFromCandidate.restype = ctypes.c_int
     l.cuttExecute.argtypes = [ctypes.c_uint, vp, vp]
     l.cuttExecute.restype = ctypes.c_int
+    l.cuttExecuteNoAlloc.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t, vp, vp, vp]
+    l.cuttExecuteNoAlloc.restype = ctypes.c_int
     l.cuttDestroy.argtypes = [ctypes.c_uint]
     l.cuttDestroy.restype = ctypes.c_int
     l.cuttGetPlanInfo.argtypes = [ctypes.c_uint, ctypes.POINTER(PlanInfo)]
@@ -169,6 +171,12 @@ def cuttPlanFromCandidate(rank, dim, permutation, sizeofType, stream, index):
 
 def cuttExecute(handle, idata, odata):
     return lib().cuttExecute(ctypes.c_uint(handle), _ptr(idata), _ptr(odata))
+
+
+def cuttExecuteNoAlloc(rank, dim, permutation, sizeofType, stream, idata, odata):
+    """Plan and execute in one call that allocates nothing on the device: returns the result code."""
+    return lib().cuttExecuteNoAlloc(int(rank), _ints(dim), _ints(permutation), int(sizeofType), _ptr(stream),
+                                    _ptr(idata), _ptr(odata))
 
 
 def cuttDestroy(handle):

@@ -423,6 +423,31 @@ cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int device
 
 }  // namespace
 
+// What cuttPlan decides for this tensor on this device: from the memory of recent decisions, or by
+// enumerating the candidates and ranking them with the cost model.  Host work only.
+static cuttResult decideHeuristically(int rank, int* dim, int* permutation, size_t sizeofType, int deviceID,
+                                      const cuttHipDeviceProps& props, Plan& chosen, int& numCandidates) {
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  const bool useCache = planCacheCapacity() > 0;
+  const std::string key = useCache ? planKey(deviceID, force, rank, dim, permutation, sizeofType) : std::string();
+  if (useCache && planCacheLookup(key, chosen, numCandidates)) return CUTT_SUCCESS;
+  std::vector<Plan> plans;
+  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
+  if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
+  refineMbarOrder(plans, props, force);
+  const int best = chooseHeuristic(plans);
+  if (best < 0) return CUTT_INTERNAL_ERROR;
+  chooseCachePolicy(plans[best], props);
+  if (useCache) planCacheInsert(key, plans[best], (int)plans.size());
+  numCandidates = (int)plans.size();
+  chosen = std::move(plans[best]);
+  return CUTT_SUCCESS;
+}
+
 static cuttResult planImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
                            size_t sizeofType, hipStream_t stream) {
   const auto t0 = std::chrono::steady_clock::now();
@@ -433,28 +458,56 @@ static cuttResult planImpl(cuttHandle* handle, int rank, int* dim, int* permutat
   int deviceID;
   cuttHipDeviceProps props;
   if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
-  int force;
-  {
-    std::lock_guard<std::mutex> lock(gMutex);
-    force = methodOverrideLocked();
+  Plan chosen;
+  int numCandidates = 0;
+  chk = decideHeuristically(rank, dim, permutation, sizeofType, deviceID, props, chosen, numCandidates);
+  if (chk != CUTT_SUCCESS) return chk;
+  return storePlan(handle, std::move(chosen), (void*)stream, deviceID, numCandidates, 0.0, t0);
+}
+
+// cuttPlan + cuttExecute in one call that allocates nothing on the device: the index tables of a
+// Packed / PackedSplit plan are built by a kernel on `stream` in the library's static scratch
+// memory, then the transpose is launched on the same stream.  See cutt.h.
+static cuttResult executeNoAllocImpl(int rank, int* dim, int* permutation, size_t sizeofType, hipStream_t stream,
+                                     void* idata, void* odata) {
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  if (chk != CUTT_SUCCESS) return chk;
+  if (idata == odata || !idata || !odata) return CUTT_INVALID_PARAMETER;
+  int deviceID;
+  cuttHipDeviceProps props;
+  if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+  Plan plan;
+  int numCandidates = 0;
+  chk = decideHeuristically(rank, dim, permutation, sizeofType, deviceID, props, plan, numCandidates);
+  if (chk != CUTT_SUCCESS) return chk;
+  plan.stream = (void*)stream;
+  plan.deviceID = deviceID;
+  void* scratch = nullptr;
+  size_t scratchBytes = 0;
+  if (plan.tableBytes() > 0) {
+    if (int e = cuttHipScratch(&scratch, &scratchBytes); e != 0) {
+      std::fprintf(stderr, "cuttExecuteNoAlloc: no address for the static scratch memory (%s)\n", cuttHipErrorString(e));
+      return CUTT_INTERNAL_ERROR;
+    }
+    if (const char* e = std::getenv("CUTT_NOALLOC_MAX_BYTES"))  // a smaller limit, for tests
+      scratchBytes = std::min(scratchBytes, (size_t)std::max(0ll, std::atoll(e)));
+    if (plan.tableBytes() > scratchBytes) {
+      std::fprintf(stderr, "cuttExecuteNoAlloc: the plan's index tables (%zu bytes) exceed the static scratch "
+                           "memory (%zu bytes)\n", plan.tableBytes(), scratchBytes);
+      return CUTT_INVALID_PARAMETER;
+    }
   }
-  const bool useCache = planCacheCapacity() > 0;
-  const std::string key = useCache ? planKey(deviceID, force, rank, dim, permutation, sizeofType) : std::string();
-  if (useCache) {
-    Plan known;
-    int numCandidates = 0;
-    if (planCacheLookup(key, known, numCandidates))
-      return storePlan(handle, std::move(known), (void*)stream, deviceID, numCandidates, 0.0, t0);
+  if (int e = plan.activateInPlace(scratch, scratchBytes); e != 0) {
+    std::fprintf(stderr, "cuttExecuteNoAlloc: building the index tables failed (%d%s%s)\n", e, e > 0 ? " " : "",
+                 e > 0 ? cuttHipErrorString(e) : "");
+    return CUTT_INTERNAL_ERROR;
   }
-  std::vector<Plan> plans;
-  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
-  if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
-  refineMbarOrder(plans, props, force);
-  const int best = chooseHeuristic(plans);
-  if (best < 0) return CUTT_INTERNAL_ERROR;
-  chooseCachePolicy(plans[best], props);
-  if (useCache) planCacheInsert(key, plans[best], (int)plans.size());
-  return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), 0.0, t0);
+  if (int e = plan.launch(idata, odata); e != 0) {
+    std::fprintf(stderr, "cuttExecuteNoAlloc: launch failed (%d%s%s)\n", e, e > 0 ? " " : "",
+                 e > 0 ? cuttHipErrorString(e) : "");
+    return CUTT_INTERNAL_ERROR;
+  }
+  return CUTT_SUCCESS;
 }
 
 static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
@@ -660,6 +713,15 @@ extern "C" cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* perm
                                size_t sizeofType, hipStream_t stream) {
   try {
     return planImpl(handle, rank, dim, permutation, sizeofType, stream);
+  } catch (...) {
+    return CUTT_INTERNAL_ERROR;
+  }
+}
+
+extern "C" cuttResult cuttExecuteNoAlloc(int rank, int* dim, int* permutation, size_t sizeofType,
+                                         hipStream_t stream, void* idata, void* odata) {
+  try {
+    return executeNoAllocImpl(rank, dim, permutation, sizeofType, stream, idata, odata);
   } catch (...) {
     return CUTT_INTERNAL_ERROR;
   }

@@ -227,6 +227,37 @@ int cuttHipValidatePacked(const cuttHipPackedArgs* args);
 int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);
+/*
+ * Index tables of one slab class built on the device (for callers that may not allocate or copy):
+ * entry i of table l is the mixed-radix sum over list[l] (first entry fastest) of index * stride;
+ * l = 0 fills rowIn (count[0] entries), l = 1 rowOut (count[1]), l = 2 the LDS gather slots
+ * (count[2] entries, stored as position + (position >> padShift)).
+ */
+typedef struct cuttHipRadixList {
+  int n;
+  uint32_t extent[CUTT_MAX_RANK];
+  uint32_t stride[CUTT_MAX_RANK];
+} cuttHipRadixList;
+
+typedef struct cuttHipTableBuildArgs {
+  uint32_t count[3];
+  int padShift;
+  cuttHipRadixList list[3];
+  uint32_t* rowIn;
+  uint32_t* rowOut;
+  uint16_t* shIdx;
+} cuttHipTableBuildArgs;
+
+int cuttHipLaunchTableBuild(const cuttHipTableBuildArgs* args, void* stream);
+
+/*
+ * The library's static scratch memory on the current device (a __device__ array in the code
+ * object, CUTT_HIP_SCRATCH_BYTES bytes, 256-byte aligned): its device address, looked up once per
+ * device.  Every caller on one device shares the same array.  0 or a hipError_t value.
+ */
+#define CUTT_HIP_SCRATCH_BYTES (1u << 20)
+int cuttHipScratch(void** ptr, size_t* bytes);
+
 /* Plain copy of `bytes` bytes (a multiple of 4) for the Trivial method; cachePolicy as above. */
 int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int cachePolicy, void* stream);
 /* One-time kernel attribute setup of the packed kernels on the current device (idempotent). */

@@ -34,6 +34,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
 #include <tuple>
 #include <type_traits>
 
@@ -654,6 +655,77 @@ extern "C" int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int ca
     case 1: return (int)launchKernel(copyKernel<1>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
     default: return (int)launchKernel(copyKernel<3>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
   }
+}
+
+// ---------------------------------------------------------------------------
+// Static scratch memory and the kernel that builds a plan's index tables in it.
+// ---------------------------------------------------------------------------
+// Device memory that exists from the moment the code object is loaded: the entry point that must
+// not allocate keeps a packed plan's index tables here.  In host code the array's name is only a
+// handle for hipGetSymbolAddress; the address it returns (one per device) is what kernels get.
+static __device__ __align__(256) unsigned char scratch[CUTT_HIP_SCRATCH_BYTES];
+
+extern "C" int cuttHipScratch(void** ptr, size_t* bytes) {
+  static std::mutex lock;
+  static void* perDevice[64] = {};
+  if (!ptr || !bytes) return (int)hipErrorInvalidValue;
+  int dev = 0;
+  if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+  if (dev < 0 || dev >= 64) return (int)hipErrorInvalidDevice;
+  std::lock_guard<std::mutex> guard(lock);
+  if (!perDevice[dev]) {
+    void* p = nullptr;
+    if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)); e != hipSuccess) return (int)e;
+    if (!p) return (int)hipErrorInvalidSymbol;
+    perDevice[dev] = p;
+  }
+  *ptr = perDevice[dev];
+  *bytes = CUTT_HIP_SCRATCH_BYTES;
+  return 0;
+}
+
+namespace {
+constexpr int kBuildThreads = 256;
+
+__device__ __forceinline__ uint32_t radixSum(const cuttHipRadixList& l, uint32_t i) {
+  uint32_t off = 0;
+  for (int k = 0; k < l.n; k++) {
+    const uint32_t q = i / l.extent[k];
+    off += (i - q * l.extent[k]) * l.stride[k];
+    i = q;
+  }
+  return off;
+}
+
+__global__ __launch_bounds__(kBuildThreads) void buildTablesKernel(const cuttHipTableBuildArgs a) {
+  const uint32_t i = blockIdx.x * kBuildThreads + threadIdx.x;
+  if (i < a.count[0]) a.rowIn[i] = radixSum(a.list[0], i);
+  if (i < a.count[1]) a.rowOut[i] = radixSum(a.list[1], i);
+  if (i < a.count[2]) {
+    const uint32_t pos = radixSum(a.list[2], i);
+    a.shIdx[i] = (uint16_t)(pos + (pos >> a.padShift));
+  }
+}
+}  // namespace
+
+extern "C" int cuttHipLaunchTableBuild(const cuttHipTableBuildArgs* a, void* stream) {
+  if (!a || !a->rowIn || !a->rowOut || !a->shIdx || a->padShift < 1 || a->padShift > 31)
+    return (int)hipErrorInvalidValue;
+  uint32_t most = 0;
+  for (int l = 0; l < 3; l++) {
+    if (a->count[l] < 1 || a->count[l] > 65536 || a->list[l].n < 0 || a->list[l].n > CUTT_MAX_RANK)
+      return (int)hipErrorInvalidValue;
+    uint64_t span = 1;  // the list must enumerate at least count entries
+    for (int k = 0; k < a->list[l].n; k++) {
+      if (a->list[l].extent[k] < 1) return (int)hipErrorInvalidValue;
+      span *= a->list[l].extent[k];
+      if (span > (1ull << 32)) return (int)hipErrorInvalidValue;
+    }
+    if (span != a->count[l]) return (int)hipErrorInvalidValue;
+    most = std::max(most, a->count[l]);
+  }
+  const dim3 grid((most + kBuildThreads - 1) / kBuildThreads), block(kBuildThreads);
+  return (int)launchKernel(buildTablesKernel, grid, block, 0, (hipStream_t)stream, *a);
 }
 
 // Lets the packed kernels use more than the default 64 KB of dynamic LDS on the current device.

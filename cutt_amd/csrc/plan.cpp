@@ -790,53 +790,65 @@ bool createPlans(const Problem& orig, const Problem& red, const cuttHipDevicePro
 }
 
 // ---------------------------------------------------------------------------
+// The mixed-radix enumerations that define the index tables of slab class c: the input offsets of
+// the contiguous input runs, the output offsets of the contiguous output runs, and for every
+// element in output-compact order its position in input-compact order (the LDS gather, before
+// padding).  False if the class geometry is inconsistent.
+static bool classRadixLists(const Plan& plan, int c, std::vector<RadixDim>& rowsIn, std::vector<RadixDim>& rowsOut,
+                            std::vector<RadixDim>& gather) {
+  const Split& sp = plan.split;
+  const Problem& pb = plan.pb;
+  const cuttHipPackedArgs& packed = plan.packed;
+  const int slab[2] = {packed.split[0].slabFloor + (c & 1), packed.split[1].slabFloor + ((c >> 1) & 1)};
+  rowsIn.clear(); rowsOut.clear(); gather.clear();
+  // Ranks of Mmk in input order with their in-compact strides.  The leading ranks up to and
+  // including the first split rank form the contiguous row; the others enumerate the rows.
+  std::vector<int64_t> compactIn(pb.rank, 0);
+  int64_t cstride = 1;
+  bool inPrefix = true;
+  for (int r = 0; r < pb.rank; r++) {
+    if (!sp.inMmk[r]) {
+      inPrefix = false;
+      continue;
+    }
+    const int e = blockExtent(sp, pb, r, slab);
+    compactIn[r] = cstride;
+    cstride *= e;
+    if (!inPrefix) rowsIn.push_back({e, pb.strideIn[r]});
+    if (sp.splitSlot(r) >= 0) inPrefix = false;  // ranks after a split rank start new rows
+  }
+  if (cstride != packed.cls[c].vol) return false;
+  // Ranks of Mmk in output order.
+  bool outPrefix = true;
+  for (int j = 0; j < pb.rank; j++) {
+    const int r = pb.perm[j];
+    if (!sp.inMmk[r]) {
+      outPrefix = false;
+      continue;
+    }
+    const int e = blockExtent(sp, pb, r, slab);
+    gather.push_back({e, compactIn[r]});
+    if (!outPrefix) rowsOut.push_back({e, pb.strideOut[r]});
+    if (sp.splitSlot(r) >= 0) outPrefix = false;
+  }
+  return true;
+}
+
 bool Plan::buildTables() {
   if (tablesBuilt) return true;
   if (method != kPacked && method != kPackedSplit) {
     tablesBuilt = true;
     return true;
   }
-  const Split& sp = split;
   for (int c = 0; c < 4; c++) {
     if (!classUsed(packed, c)) continue;
-    const int slab[2] = {packed.split[0].slabFloor + (c & 1), packed.split[1].slabFloor + ((c >> 1) & 1)};
     PackedTables& t = tab[c];
     t.vol = packed.cls[c].vol;
     t.inCont = packed.cls[c].inCont;
     t.outCont = packed.cls[c].outCont;
-    // Ranks of Mmk in input order with their in-compact strides.  The leading ranks up to and
-    // including the first split rank form the contiguous row; the others enumerate the rows.
-    std::vector<int64_t> compactIn(pb.rank, 0);
-    int64_t cstride = 1;
-    std::vector<RadixDim> rowsIn;
-    bool inPrefix = true;
-    for (int r = 0; r < pb.rank; r++) {
-      if (!sp.inMmk[r]) {
-        inPrefix = false;
-        continue;
-      }
-      const int e = blockExtent(sp, pb, r, slab);
-      compactIn[r] = cstride;
-      cstride *= e;
-      if (!inPrefix) rowsIn.push_back({e, pb.strideIn[r]});
-      if (sp.splitSlot(r) >= 0) inPrefix = false;  // ranks after a split rank start new rows
-    }
-    if (cstride != t.vol) return false;
+    std::vector<RadixDim> rowsIn, rowsOut, gather;
+    if (!classRadixLists(*this, c, rowsIn, rowsOut, gather)) return false;
     enumerateOffsets(rowsIn, t.vol / t.inCont, t.rowIn);
-    // Ranks of Mmk in output order.
-    std::vector<RadixDim> rowsOut, gather;
-    bool outPrefix = true;
-    for (int j = 0; j < pb.rank; j++) {
-      const int r = pb.perm[j];
-      if (!sp.inMmk[r]) {
-        outPrefix = false;
-        continue;
-      }
-      const int e = blockExtent(sp, pb, r, slab);
-      gather.push_back({e, compactIn[r]});
-      if (!outPrefix) rowsOut.push_back({e, pb.strideOut[r]});
-      if (sp.splitSlot(r) >= 0) outPrefix = false;
-    }
     enumerateOffsets(rowsOut, t.vol / t.outCont, t.rowOut);
     std::vector<uint32_t> pos;
     enumerateOffsets(gather, t.vol, pos);
@@ -845,6 +857,67 @@ bool Plan::buildTables() {
   }
   tablesBuilt = true;
   return true;
+}
+
+// Layout of a plan's tables in one piece of device memory: [rowIn | rowOut | shIdx] per class,
+// each piece 16-byte aligned.  Returns the total size.
+static size_t tableLayout(const cuttHipPackedArgs& packed, size_t off[4][3]) {
+  auto align16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
+  size_t total = 0;
+  for (int c = 0; c < 4; c++) {
+    off[c][0] = off[c][1] = off[c][2] = 0;
+    if (!classUsed(packed, c)) continue;
+    const cuttHipPackedClass& k = packed.cls[c];
+    off[c][0] = total; total += align16((size_t)(k.vol / k.inCont) * sizeof(uint32_t));
+    off[c][1] = total; total += align16((size_t)(k.vol / k.outCont) * sizeof(uint32_t));
+    off[c][2] = total; total += align16((size_t)k.vol * sizeof(uint16_t));
+  }
+  return total;
+}
+
+size_t Plan::tableBytes() const {
+  if (method != kPacked && method != kPackedSplit) return 0;
+  size_t off[4][3];
+  return tableLayout(packed, off);
+}
+
+int Plan::activateInPlace(void* tables, size_t capacity) {
+  if (method != kPacked && method != kPackedSplit) return activate();
+  if (dTables || !tables) return -1;
+  size_t off[4][3];
+  if (tableLayout(packed, off) > capacity) return -1;
+  if (int e = cuttHipPreparePacked(); e != 0) return e;
+  unsigned char* base = (unsigned char*)tables;
+  for (int c = 0; c < 4; c++) {
+    if (!classUsed(packed, c)) continue;
+    std::vector<RadixDim> lists[3];
+    if (!classRadixLists(*this, c, lists[0], lists[1], lists[2])) return -1;
+    cuttHipTableBuildArgs b;
+    std::memset(&b, 0, sizeof(b));
+    const cuttHipPackedClass& k = packed.cls[c];
+    b.count[0] = (uint32_t)(k.vol / k.inCont);
+    b.count[1] = (uint32_t)(k.vol / k.outCont);
+    b.count[2] = (uint32_t)k.vol;
+    b.padShift = packed.padShift;
+    for (int l = 0; l < 3; l++) {
+      if ((int)lists[l].size() > CUTT_MAX_RANK) return -1;
+      b.list[l].n = (int)lists[l].size();
+      for (int i = 0; i < b.list[l].n; i++) {
+        b.list[l].extent[i] = (uint32_t)lists[l][i].extent;
+        b.list[l].stride[i] = (uint32_t)lists[l][i].stride;
+      }
+    }
+    b.rowIn = (uint32_t*)(base + off[c][0]);
+    b.rowOut = (uint32_t*)(base + off[c][1]);
+    b.shIdx = (uint16_t*)(base + off[c][2]);
+    if (int e = cuttHipLaunchTableBuild(&b, stream); e != 0) return e;
+    packed.cls[c].rowIn = b.rowIn;
+    packed.cls[c].rowOut = b.rowOut;
+    packed.cls[c].shIdx = b.shIdx;
+  }
+  if (int v = cuttHipValidatePacked(&packed); v != 0) return v;
+  launchable = true;
+  return 0;
 }
 
 int Plan::activate() {
@@ -857,16 +930,8 @@ int Plan::activate() {
   if (dTables) return 0;
   if (!buildTables()) return -1;
   if (int e = cuttHipPreparePacked(); e != 0) return e;
-  // One allocation: [rowIn | rowOut | shIdx] per class, each piece 16-byte aligned.
-  auto align16 = [](size_t v) { return (v + 15) & ~(size_t)15; };
-  size_t total = 0;
-  size_t off[4][3] = {};
-  for (int c = 0; c < 4; c++) {
-    if (!classUsed(packed, c)) continue;
-    off[c][0] = total; total += align16(tab[c].rowIn.size() * sizeof(uint32_t));
-    off[c][1] = total; total += align16(tab[c].rowOut.size() * sizeof(uint32_t));
-    off[c][2] = total; total += align16(tab[c].shIdx.size() * sizeof(uint16_t));
-  }
+  size_t off[4][3];
+  const size_t total = tableLayout(packed, off);
   std::vector<unsigned char> host(total, 0);
   for (int c = 0; c < 4; c++) {
     if (!classUsed(packed, c)) continue;
@@ -909,7 +974,6 @@ int Plan::launch(const void* in, void* out) {
       return cuttHipLaunchTiledCopy(&tcopy, in, out, stream);
     case kPacked:
     case kPackedSplit:
-      if (!dTables) return -1;
       return cuttHipLaunchPacked(&packed, in, out, stream);
     default:
       return -1;

@@ -122,6 +122,11 @@ struct Plan {
   Plan clone() const;             // host-side copy of a plan that has no device tables yet
   bool buildTables();             // Packed/PackedSplit: fill tab[]; others: no-op
   int activate();                 // upload tables, check the launch arguments; 0 or an error code
+  // Like activate(), but the tables are built by a kernel on `stream` in device memory the caller
+  // provides (`capacity` bytes, 16-byte aligned) instead of being allocated and uploaded; the plan
+  // does not own that memory.  Nothing is allocated on the device.
+  int activateInPlace(void* tables, size_t capacity);
+  size_t tableBytes() const;      // device bytes of the index tables (0 for methods without)
   int launch(const void* in, void* out);  // asynchronous on stream
   void release();                 // free device tables
   std::string describe() const;

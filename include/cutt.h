@@ -86,6 +86,25 @@ cuttResult cuttDestroy(cuttHandle handle);
  */
 cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata);
 
+/*
+ * Plan and execute in one call without allocating anything on the device.  No counterpart in the
+ * reference; it is for callers that cannot allocate device memory where they transpose (tight
+ * serving loops, harnesses that forbid hipMalloc): cuttPlan allocates a Packed / PackedSplit
+ * plan's index tables with hipMalloc and copies them to the device, this call builds them with a
+ * kernel on `stream` in static device memory of the library (1 MiB per GPU, held until the
+ * process ends) and launches the same transpose kernel after it on `stream`.  The plan is the
+ * one cuttPlan would choose; arguments and checks are those of cuttPlan and cuttExecute.
+ *
+ * Limits: a plan whose index tables exceed the static memory is refused with
+ * CUTT_INVALID_PARAMETER and a message on stderr (the tables of the plans this library builds
+ * need at most 640 KiB).  Every call on one GPU uses the same static memory: calls on the same
+ * stream are ordered and safe, calls whose work may overlap on the GPU (different streams, several
+ * host threads) race and must be serialised by the caller.  The memory keeps the last call's
+ * tables; every entry a call uses is rewritten by that call, nothing needs to start at zero.
+ */
+cuttResult cuttExecuteNoAlloc(int rank, int* dim, int* permutation, size_t sizeofType,
+                              hipStream_t stream, void* idata, void* odata);
+
 #ifdef __cplusplus
 }
 #endif

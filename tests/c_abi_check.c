@@ -25,6 +25,9 @@ int main(void) {
   if (cuttPlan(&h, 3, dim, bad, 8, 0) != CUTT_INVALID_PARAMETER) return 13;
   if (cuttPlan(0, 3, dim, perm, 8, 0) != CUTT_INVALID_PARAMETER) return 14;
   if (cuttPlanMeasure(&h, 3, dim, perm, 8, 0, (void*)dim, (void*)dim) != CUTT_INVALID_PARAMETER) return 15;
+  if (cuttExecuteNoAlloc(3, dim, perm, 3, 0, (void*)dim, (void*)perm) != CUTT_INVALID_PARAMETER) return 27;
+  if (cuttExecuteNoAlloc(3, dim, bad, 8, 0, (void*)dim, (void*)perm) != CUTT_INVALID_PARAMETER) return 28;
+  if (cuttExecuteNoAlloc(3, dim, perm, 8, 0, (void*)dim, (void*)dim) != CUTT_INVALID_PARAMETER) return 29;
   if (cuttExecute(123456u, (void*)dim, (void*)perm) != CUTT_INVALID_PLAN) return 16;
   if (cuttDestroy(123456u) != CUTT_INVALID_PLAN) return 17;
   if (cuttGetPlanInfo(123456u, &info) != CUTT_INVALID_PLAN) return 18;
