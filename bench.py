@@ -28,10 +28,19 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 import numpy as np
 
 HBM_PEAK_GBS = 8000.0
-# HBM bytes per launch of the C2 transpose kernel from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE
+# HBM bytes per launch of the C2 transpose kernel, from rocprofv3 counters (FETCH_SIZE and WRITE_SIZE
 # in runs of their own, each scaled by what the counter reads for the same-size device-to-device
-# copy): 1 610 695 680 fetched + 1 611 192 627 written.  Only valid for the Tiled plan of C2.
-C2_TILED_TRAFFIC_BYTES = 3221888307
+# copy).  A figure belongs to one launched kernel instance: it is reported only when the plan of
+# this run has the signature (method, workgroups, tile order, super-tile shape, cache policy, rows
+# in groups) the profile was taken on, together with the name of the profile; otherwise null.
+C2_TRAFFIC_PROFILES = {
+    ("Tiled", 49152, 5, 8, 16, 3, 0): (3221890765, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
+}
+
+
+def plan_signature(info):
+    return (info.method_name, int(info.numBlocks), int(info.tiledOrder), int(info.superM), int(info.superK),
+            int(info.cachePolicy), int(info.tiledGrouped))
 
 
 def log(*a):
@@ -145,7 +154,8 @@ def cpu_baseline(cfg, data, budget_s=20.0):
     import oracle
     dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
     nbytes = data.size * es
-    cores = min(16, os.cpu_count() or 1)
+    host_cores = os.cpu_count() or 1
+    cores = min(16, host_cores)
     out = np.empty_like(data)
     best = None
     t_start = time.perf_counter()
@@ -156,7 +166,7 @@ def cpu_baseline(cfg, data, budget_s=20.0):
         dt = time.perf_counter() - t0
         best = dt if best is None else min(best, dt)
         reps += 1
-    return dict(value=round(2.0 * nbytes / best / 1e9, 2), unit="GB/s", cores=cores, kind="port",
+    return dict(value=round(2.0 * nbytes / best / 1e9, 2), unit="GB/s", cores=cores, host_cores=host_cores, kind="port",
                 sample="%d full passes of the same workload (%s, %d elements), best pass" % (reps, cfg["name"], data.size),
                 note="the reference has no CPU transpose; this is the oracle's multithreaded C port")
 
@@ -200,13 +210,9 @@ def main():
             with open(os.path.join(args.out, "bench_all.json"), "w") as f:
                 json.dump(results, f, indent=1)
         if args.sweep:
-            sres = []
-            for cfg in bc.sweep()[: args.sweep]:
-                data = bc.make_input(cfg, seed=5)
-                for how in ("plan", "measure"):
-                    res = r.run_config(cfg, how, data=data, reps=4)
-                    log(json.dumps(res))
-                    sres.append(res)
+            import sweep_runner
+            sres = [sweep_runner.run_tensor(cfg, reps=4, log=log) for cfg in bc.sweep()[: args.sweep]]
+            log(sweep_runner.table(sres))
             with open(os.path.join(args.out, "bench_sweep.json"), "w") as f:
                 json.dump(sres, f, indent=1)
         return
@@ -251,7 +257,6 @@ def main():
     bit_exact = bool(np.array_equal(d_out.cpu().numpy().view(data.dtype), expect))
     if not bit_exact:
         raise SystemExit("bench output differs from the CPU oracle")
-    c.cuttDestroy(h)
 
     # the same workload through the measuring planner (reported beside the contract value)
     hm, plan_ms_m = r.plan(cfg, "measure", d_in, d_out)
@@ -259,10 +264,27 @@ def main():
     ms_m = r.time_calls(lambda: c.cuttExecute(hm, d_in.data_ptr(), d_out.data_ptr()), 8, out=d_out)
     c.cuttDestroy(hm)
 
+    # the same-size device-to-device copy, timed both ways: like the timed region above (K calls back
+    # to back, wall clock) and with the reference's per-call protocol (output fill, synchronise,
+    # event-timed call; best of 8)
+    def copy_step():
+        assert r.lib.cuttHipMemcpyDtoDAsync(d_out.data_ptr(), d_in.data_ptr(), nbytes, r.stream) == 0
+    for _ in range(args.warmup):
+        copy_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        copy_step()
+    torch.cuda.synchronize()
+    copy_wall = time.perf_counter() - t0
+    memcpy_gbs_loop = 2.0 * nbytes / (copy_wall / args.steps) / 1e9
     cp = r.memcpy_ms(d_in, d_out)
     memcpy_gbs = effective_gbs(nbytes, min(cp))
+    exec_ms = r.time_calls(step, 8, out=d_out)   # the transpose with the per-call protocol
+    c.cuttDestroy(h)
     value = 2.0 * nbytes / (wall / args.steps) / 1e9
     achieved = 2.0 * nbytes / (avg_kernel_ms * 1e-3) / 1e9
+    traffic, traffic_source = C2_TRAFFIC_PROFILES.get(plan_signature(info), (None, None))
     line = {
         "metric": "effective transpose bandwidth GB/s (2×bytes/time) and % of D2D memcpy, 1 GPU",
         "value": round(value, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -270,15 +292,20 @@ def main():
         "dtype": "u64", "data": "synthetic",
         "config": {"workload": "C2: fp64 dims (1024,64,1024,3) perm (2,1,0,3), 201326592 elements, value = linear index",
                    "planner": "cuttPlan", "method": info.method_name, "blocks": info.numBlocks,
-                   "threads": info.numThreads, "plan_ms": round(plan_ms, 2)},
-        "pct_of_d2d_memcpy": round(100.0 * value / memcpy_gbs, 1),
-        "d2d_memcpy_GBs": round(memcpy_gbs, 1),
+                   "threads": info.numThreads, "tile_order": info.tiledOrder, "super_tile": [info.superM, info.superK],
+                   "cache_policy": info.cachePolicy, "plan_ms": round(plan_ms, 2)},
+        "pct_of_d2d_memcpy": round(100.0 * value / memcpy_gbs_loop, 1),
+        "d2d_memcpy_GBs": round(memcpy_gbs_loop, 1),
+        "per_call_protocol": {"transpose_GBs_best": round(effective_gbs(nbytes, min(exec_ms)), 1),
+                              "d2d_memcpy_GBs_best": round(memcpy_gbs, 1),
+                              "pct_of_d2d_memcpy": round(100.0 * min(cp) / min(exec_ms), 1),
+                              "what": "output fill + synchronise + one event-timed call, best of 8 (reference src/cutt_bench.cpp:818-827)"},
         "bit_exact_vs_cpu_oracle": bit_exact,
         "cuttPlanMeasure": {"GBs_best": round(effective_gbs(nbytes, min(ms_m)), 1), "method": info_m.method_name,
                             "plan_ms": round(plan_ms_m, 1)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": C2_TILED_TRAFFIC_BYTES if info.method_name == "Tiled" else None,
+                     "traffic": traffic, "traffic_source": traffic_source,
                      "kernel_ms_avg": round(avg_kernel_ms, 4), "algorithmic_bytes": 2 * nbytes},
     }
     if not args.no_cpu:

@@ -51,7 +51,7 @@ class PlanInfo(ctypes.Structure):
         ("numCandidates", ctypes.c_int), ("planMs", ctypes.c_double),
         ("cachePolicy", ctypes.c_int), ("elemsPerThread", ctypes.c_int),
         ("rdEdgeDist", ctypes.c_double), ("wrEdgeDist", ctypes.c_double),
-        ("tiledGrouped", ctypes.c_int),
+        ("tiledGrouped", ctypes.c_int), ("superM", ctypes.c_int), ("superK", ctypes.c_int),
     ]
 
     @property

@@ -201,6 +201,8 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
                                       : (p.method == kTiledCopy ? p.tcopy.cachePolicy : p.packed.cachePolicy);
   o.elemsPerThread = p.packed.elemsPerThread;
   o.tiledGrouped = p.method == kTiled ? p.tiled.grouped : 0;
+  o.superM = p.method == kTiled ? (int)p.tiled.superM : (p.method == kTiledCopy ? (int)p.tcopy.superM : 0);
+  o.superK = p.method == kTiled ? (int)p.tiled.superK : (p.method == kTiledCopy ? (int)p.tcopy.superK : 0);
   o.rdEdgeDist = p.model.rdEdgeDist;
   o.wrEdgeDist = p.model.wrEdgeDist;
 }

@@ -55,6 +55,7 @@ typedef struct cuttPlanInfo {
    * runs, on the read and on the write side (0 = no such neighbour) */
   double rdEdgeDist, wrEdgeDist;
   int tiledGrouped;     /* Tiled: 1 if a lane keeps 4 instead of 16 tile rows in flight */
+  int superM, superK;   /* Tiled/TiledCopy: shape of the super-tiles the workgroups walk (tiled orders 3-5) */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */

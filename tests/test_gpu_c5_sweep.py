@@ -1,0 +1,67 @@
+"""The whole sweep configuration: 50 seeded random tensors of about 2e8 elements, ranks 2-7, 8- and
+4-byte elements alternating, every one planned with cuttPlan and with cuttPlanMeasure, timed with
+the reference's protocol beside a same-size device-to-device copy, every output checked on the
+device against torch's permute of the index pattern, six of them also against the CPU oracle on
+random bits.  The target - every 8-byte tensor at 70 % of the copy or better - is asserted for both
+planners; plan-creation times are reported."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+import baseline_configs as bc
+
+pytestmark = pytest.mark.gpu
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+
+
+def say(msg):
+    print(msg, flush=True)
+    sys.stdout.flush()
+
+
+def test_sweep_both_planners_every_tensor():
+    import torch
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    import cutt_amd
+    import sweep_runner
+    cutt_amd.lib()
+    cutt_amd.set_method_override(0)
+    results = []
+    for cfg in bc.sweep():
+        results.append(sweep_runner.run_tensor(cfg, reps=4, log=say))
+    text = sweep_runner.table(results)
+    say(text)
+    out_dir = os.path.join(ROOT, "gpurun_out")
+    if os.path.isdir(out_dir):
+        with open(os.path.join(out_dir, "c5_sweep_table.txt"), "w") as f:
+            f.write(text + "\n")
+    assert len(results) == 50
+    for r in results:
+        for how in ("plan", "measure"):
+            assert r[how]["exact"], (r["name"], how)
+    fp64 = [r for r in results if r["es"] == 8]
+    worst_measured = min(fp64, key=lambda r: r["measure"]["pct"])
+    worst_heuristic = min(fp64, key=lambda r: r["plan"]["pct"])
+    assert worst_measured["measure"]["pct"] >= 70.0, worst_measured
+    assert worst_heuristic["plan"]["pct"] >= 70.0, worst_heuristic
+    # the measuring planner must not end up behind the heuristic one by more than timing noise
+    for r in results:
+        assert r["measure"]["ms"] <= 1.08 * r["plan"]["ms"], r
+
+
+@pytest.mark.parametrize("index", [0, 9, 18, 27, 36, 45])
+def test_sweep_tensor_against_cpu_oracle(index):
+    import gpu_util
+    import oracle
+    cfg = bc.sweep()[index]
+    dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
+    data = bc.make_input(cfg, seed=77 + index)
+    say("%s dim=%s perm=%s es=%d: oracle on the host" % (cfg["name"], dim, perm, es))
+    expect = oracle.transpose_mt(dim, perm, data, 16)
+    for how in ("plan", "measure"):
+        say("%s %s" % (cfg["name"], how))
+        gpu_util.check_case(dim, perm, es, data=data, how=how, expect=expect)

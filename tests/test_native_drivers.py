@@ -65,6 +65,32 @@ def test_cutt_bench_ttc_suite():
     assert r.stdout.count("number of elements") == 57
 
 
+def _suite_summary(out):
+    """(tensors, min % of memcpy) from the driver's closing line."""
+    import re
+    m = re.search(r"percent of same-size hipMemcpy .*: tensors (\d+) min ([0-9.]+) median ([0-9.]+)", out)
+    assert m, out[-2000:]
+    return int(m.group(1)), float(m.group(2)), float(m.group(3))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("planner", ["heuristic", "measure"])
+def test_cutt_bench_random_suites_short(planner):
+    # the reference's random-tensor suites with two tensors per rank (or per shape) instead of 50 / 500:
+    # bench 3 (ranks 2-8 and 15, reference src/cutt_bench.cpp:414-431), bench 5 with extent ratio 10
+    # (ranks 2-7, :455-546) and bench 7 (ranks 8 and 12 with four large extents, :688-728); every
+    # tensor is checked on the device, and the 8-byte suites must stay above 70 % of the same-size copy
+    extra = ["-measure"] if planner == "measure" else []
+    for bench, tensors in (("3", 16), ("510", 12), ("7", 6)):
+        r = run("cutt_bench", "-bench", bench, "-samples", "2", "-seed", "11", "-plantimer", *extra, timeout=600)
+        assert r.returncode == 0, r.stdout[-2000:]
+        assert "bench OK" in r.stdout and "plan took" in r.stdout
+        n, worst, median = _suite_summary(r.stdout)
+        print("bench %s %s: %d tensors, %% of memcpy min %.1f median %.1f" % (bench, planner, n, worst, median), flush=True)
+        assert n >= tensors - 2   # bench 7 skips a shuffle that happens to be the identity
+        assert worst >= 70.0, r.stdout[-3000:]
+
+
 @pytest.mark.gpu
 def test_tensor_above_4GB_uses_wide_offsets():
     # 671 088 640 doubles = 5.4 GB per buffer: byte offsets no longer fit 32 bits
