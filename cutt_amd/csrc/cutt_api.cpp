@@ -390,8 +390,8 @@ PlannerOptions plannerOptions(int forceMethod) {
   }
   if (const char* e = std::getenv("CUTT_WIDE_OFFSETS")) opt.wideOffsets = std::atoi(e) != 0;
   if (const char* e = std::getenv("CUTT_MBAR_ORDER")) opt.mbarOrder = std::atoi(e);
-  if (const char* e = std::getenv("CUTT_SUPER_M")) opt.superM = std::max(1, std::atoi(e));
-  if (const char* e = std::getenv("CUTT_SUPER_K")) opt.superK = std::max(1, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_SUPER_M")) { opt.superM = std::max(1, std::atoi(e)); opt.superAuto = false; }
+  if (const char* e = std::getenv("CUTT_SUPER_K")) { opt.superK = std::max(1, std::atoi(e)); opt.superAuto = false; }
   if (const char* e = std::getenv("CUTT_TILED_GROUPED")) opt.tiledGrouped = std::atoi(e) != 0 ? 1 : 0;
   return opt;
 }
@@ -603,8 +603,15 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
     // options that reproduce the winner as it stands
     PlannerOptions cur = plannerOptions(force);
     cur.cachePolicy = cachePolicyOf(plans[best]);
-    if (tiled) cur.tiledOrder = plans[best].method == kTiled ? plans[best].tiled.order : plans[best].tcopy.order;
-    else cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
+    if (tiled) {
+      const bool t = plans[best].method == kTiled;
+      cur.tiledOrder = t ? plans[best].tiled.order : plans[best].tcopy.order;
+      cur.superM = (int)(t ? plans[best].tiled.superM : plans[best].tcopy.superM);
+      cur.superK = (int)(t ? plans[best].tiled.superK : plans[best].tcopy.superK);
+      cur.superAuto = false;
+    } else {
+      cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
+    }
     if (plans[best].method == kTiled) cur.tiledGrouped = plans[best].tiled.grouped;
     const PlannerOptions start = cur;
 
@@ -632,11 +639,11 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
       // along Mm / along Mk, strips per Mbar position / for all Mbar positions in turn
       struct TileKnob { int order, superM, superK; };
       for (const TileKnob& k : {TileKnob{5, 16, 16}, TileKnob{5, 2, 8}, TileKnob{5, 8, 2}, TileKnob{5, 32, 2},
-                                TileKnob{1, start.superM, start.superK},
-                                TileKnob{2, start.superM, start.superK}, TileKnob{3, start.superM, start.superK},
-                                TileKnob{5, start.superM, start.superK}}) {
+                                TileKnob{5, 4, 8}, TileKnob{5, 8, 8}, TileKnob{5, 8, 4096}, TileKnob{5, 4, 4096},
+                                TileKnob{1, 8, 4096}, TileKnob{2, 8, 4096}, TileKnob{3, 8, 4096},
+                                TileKnob{3, 16, 16}}) {
         if (failed) break;
-        if (k.order == start.tiledOrder && k.superM == start.superM) continue;
+        if (k.order == start.tiledOrder && k.superM == start.superM && k.superK == start.superK) continue;
         PlannerOptions v = cur;
         v.tiledOrder = k.order; v.superM = k.superM; v.superK = k.superK;
         if (tryVariant(v, false)) cur = v;

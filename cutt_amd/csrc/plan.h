@@ -136,6 +136,7 @@ struct PlannerOptions {
   int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
   int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3-5: strips of 8 tiles along Mm
+  bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
