@@ -81,7 +81,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
@@ -298,7 +298,7 @@ bool parallelFor(int n, F&& f) {
 // 0.3-0.5 GB; outside these limits the same switch costs up to 14 % (aligned or cache-sized
 // tensors, 8-byte elements).  (Not applied when CUTT_TILED_GROUPED pins the switch.)
 void chooseTiledGrouping(Plan& p, const cuttHipDeviceProps& props) {
-  if (p.method != kTiled || std::getenv("CUTT_TILED_GROUPED")) return;
+  if (p.method != kTiled || std::getenv("CUTT_TILED_GROUPED") || p.tiled.alignedStores) return;
   const double bytes = (double)p.pb.volume * p.pb.elemSize;
   const double lines = bytes / 128.0;
   const double cache = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
@@ -393,6 +393,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_SUPER_M")) { opt.superM = std::max(1, std::atoi(e)); opt.superAuto = false; }
   if (const char* e = std::getenv("CUTT_SUPER_K")) { opt.superK = std::max(1, std::atoi(e)); opt.superAuto = false; }
   if (const char* e = std::getenv("CUTT_TILED_GROUPED")) opt.tiledGrouped = std::atoi(e) != 0 ? 1 : 0;
+  if (const char* e = std::getenv("CUTT_TILED_ALIGNED")) opt.tiledAligned = std::atoi(e) != 0 ? 1 : 0;
   return opt;
 }
 

@@ -26,6 +26,10 @@ extern "C" {
 /* Largest tensor rank the kernels accept (the per-rank tables travel as kernel arguments). */
 #define CUTT_MAX_RANK 32
 
+/* A launch's workgroups x lanes per workgroup must fit the dispatch packet's 32-bit count of
+ * work-items; a larger grid is not refused by the runtime but silently truncated. */
+#define CUTT_HIP_MAX_GRID_LANES 0xffffffffull
+
 /* Device facts the planner and the cost model need. */
 typedef struct cuttHipDeviceProps {
   int cuCount;              /* compute units */
@@ -110,6 +114,9 @@ typedef struct cuttHipTiledArgs {
   int cachePolicy;    /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
   int grouped;        /* 0: a lane has all 16 rows of its tile in flight at once; 1: four at a time
                          (each group of 16 tile rows is waited for before the next is requested) */
+  int alignedStores;  /* 1: every tile row stores its own 64-element window of the output run, shifted
+                         so that it starts on a 128-byte line; tilesK is then
+                         ceil((volMk + 128/elemSize - 1) / 64) and grouped must be 0 */
   cuttHipMbar mbar;
 } cuttHipTiledArgs;
 

@@ -40,6 +40,7 @@
 
 #include "hip_layer.h"
 #include "mbar_decode.h"
+#include "tile_order.h"
 
 using namespace cutt;
 
@@ -63,78 +64,6 @@ __device__ __forceinline__ void stg(T* p, T v) {
 // Blocks the wave until its outstanding global loads have returned and its stores have been
 // acknowledged (the vector memory counter reaches zero); also a barrier for the compiler.
 __device__ __forceinline__ void waitForGlobalAccesses() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
-
-constexpr int kTile = 64;             // tile edge in elements
-constexpr int kTileThreads = 256;     // 4 wavefronts
-constexpr int kTileRows = kTile * kTile / kTileThreads;  // rows per lane: 16
-constexpr int kGroupRows = 4;                            // rows per lane in one skippable group
-constexpr int kRowGroups = kTileRows / kGroupRows;       // 4 groups of 16 tile rows each
-constexpr int kWaves = kTileThreads / 64;
-
-// Workgroup index -> (tile along Mm, tile along Mk, Mbar position).  Returns false for the
-// padding workgroups of order 3.
-//
-// The chip has 8 XCDs with private L2s and hands workgroup b to XCD b % 8, so neighbouring
-// tiles - which share the 128-byte lines at their unaligned edges - would otherwise always land
-// in different L2s.  With xcdChunk != 0, XCD x walks its own contiguous chunk of the logical
-// sequence.  Orders 0-2 number the logical sequence with the Mbar position, the tile along Mm or
-// the tile along Mk running fastest; orders 3 and 4 visit the tiles in superM x superK super-tiles, so
-// that both the read neighbours (along Mm) and the write neighbours (along Mk) of a tile are
-// resident in the same L2 at about the same time.  Order 5 is order 3 with the Mbar position running
-// between the super-tiles: the runs of consecutive Mbar positions, which are neighbours in memory
-// when the fastest Mbar rank follows Mk in the output (or Mm in the input), then meet in the L2 too.
-constexpr uint32_t kNumXcd = 8;
-
-struct TileOrder {
-  int order;
-  uint32_t xcdChunk, superM, superK;
-};
-
-__device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint32_t tilesM,
-                                           uint32_t tilesK, uint32_t volMbar, uint32_t& tm,
-                                           uint32_t& tk, uint32_t& m) {
-  const uint32_t l = o.xcdChunk ? (bid % kNumXcd) * o.xcdChunk + bid / kNumXcd : bid;
-  if (o.order == 0) {
-    const uint32_t t = l / volMbar;
-    m = l - t * volMbar;
-    tk = t / tilesM;
-    tm = t - tk * tilesM;
-    return tk < tilesK;
-  } else if (o.order == 1) {
-    const uint32_t t = l / tilesM;
-    tm = l - t * tilesM;
-    m = t / tilesK;
-    tk = t - m * tilesK;
-    return m < volMbar;
-  } else if (o.order == 2) {
-    const uint32_t t = l / tilesK;
-    tk = l - t * tilesK;
-    m = t / tilesM;
-    tm = t - m * tilesM;
-    return m < volMbar;
-  }
-  const uint32_t nSuperM = (tilesM + o.superM - 1) / o.superM, nSuperK = (tilesK + o.superK - 1) / o.superK;
-  const uint32_t per = o.superM * o.superK;
-  const uint32_t w = l % per;
-  const uint32_t t = l / per;
-  uint32_t st;
-  if (o.order == 5) {  // like 3, but a super-tile is visited for every Mbar position in turn
-    st = t / volMbar;
-    m = t - st * volMbar;
-    if (st >= nSuperM * nSuperK) return false;
-  } else {
-    st = t % (nSuperM * nSuperK);
-    m = t / (nSuperM * nSuperK);
-  }
-  if (o.order != 4) {  // inside a super-tile the tiles along Mm run fastest
-    tm = (st % nSuperM) * o.superM + (w % o.superM);
-    tk = (st / nSuperM) * o.superK + (w / o.superM);
-  } else {             // order 4: the tiles along Mk run fastest, super-tiles advance along Mk first
-    tk = (st % nSuperK) * o.superK + (w % o.superK);
-    tm = (st / nSuperK) * o.superM + (w / o.superK);
-  }
-  return m < volMbar && tm < tilesM && tk < tilesK;
-}
 
 // ---------------------------------------------------------------------------
 // Tiled: 64x64 tile through padded LDS.
@@ -243,6 +172,102 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
             stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
           }
         }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Tiled with line-aligned stores.  When the output rows (runs along Mk) start off the 128-byte
+// grid, the 64-wide store of a tile row covers three lines, two of them partly, and the tile next
+// door along Mk completes them later.  Here every row of a tile takes its own window of 64
+// elements along Mk: row m, whose output run starts s_m elements past a line boundary, stores the
+// elements [64 tk - s_m, 64 tk - s_m + 64) of its run, so every store of a wave is two whole lines
+// (except at the two ends of a run).  The windows of the rows of a tile differ by up to one line,
+// so the workgroup reads up to 64 + (elements per line - 1) rows along Mk into a taller LDS tile;
+// the rows in the fringe are also read by the tile next door (from the L2).  The grid has
+// ceil((volMk + elements per line - 1) / 64) tiles along Mk.
+template <typename T>
+constexpr int kLineElems = 128 / (int)sizeof(T);
+template <typename T>
+constexpr int kAlignedRows = kTile + kLineElems<T> - 1;  // rows along Mk that a workgroup may need
+
+template <typename T, int NT>
+__global__ __launch_bounds__(kTileThreads) void tiledAlignedKernel(const cuttHipTiledArgs a,
+                                                                   const T* __restrict__ in,
+                                                                   T* __restrict__ out) {
+  constexpr int LE = kLineElems<T>;
+  constexpr int ROWS = kAlignedRows<T>;
+  constexpr int RD = (ROWS + kWaves - 1) / kWaves;  // rows a wave reads at most
+  __shared__ T tile[ROWS][kTile + 1];
+
+  uint32_t tm, tk, m;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  uint32_t offIn, offOut;
+  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t m0 = tm * kTile;
+  const int32_t kBase = (int32_t)(tk * kTile) - (LE - 1);  // first row along Mk the tile may need
+  const uint32_t volMm = a.volMm, volMk = a.volMk;
+  const uint32_t wM = min((uint32_t)kTile, volMm - m0) - 1;
+  const uint32_t groupsM = (wM >> 4) + 1;
+
+  // Misalignment of output row m in elements (the low bits of its element address).  Over the
+  // rows of a tile it takes the values c + j g (mod LE), g = gcd(strideOutM, LE): the rows along
+  // Mk that some row of the tile needs are kBase + [LE - 1 - sMax, LE - 1 - sMin + 64).
+  const uint32_t outWord = (uint32_t)(reinterpret_cast<uintptr_t>(out) / sizeof(T)) + offOut;
+  const uint32_t g = min((uint32_t)LE, a.strideOutM & (0u - a.strideOutM));  // lowest set bit, capped
+  const uint32_t sMin = (outWord + m0 * a.strideOutM) & (g - 1);
+  const uint32_t sMax = sMin + (LE - g);
+  const uint32_t rowLo = (LE - 1) - sMax, rowHi = (LE - 1) - sMin + kTile;  // [rowLo, rowHi)
+
+  // Read: lanes run along input rank 0, rows along Mk (clamped to the rank's ends).
+  {
+    const uint32_t cx = min(lane, wM);
+    const T* src = in + (offIn + m0 + cx);
+    T v[RD];
+#pragma unroll
+    for (int j = 0; j < RD; j++) {
+      const uint32_t row = wave + kWaves * j;
+      if (row >= rowLo && row < rowHi) {  // uniform over the wave
+        const int32_t k = min(max(kBase + (int32_t)row, 0), (int32_t)volMk - 1);
+        v[j] = ldg<NT>(src + (uint32_t)k * a.strideInK);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < RD; j++) {
+      const uint32_t row = wave + kWaves * j;
+      if (row >= rowLo && row < rowHi) tile[row][cx] = v[j];
+    }
+  }
+  __syncthreads();
+  // Write: lanes run along Mk inside the row's own window.
+  {
+    T v[kTileRows];
+    uint32_t dstOff[kTileRows];
+#pragma unroll
+    for (int gI = 0; gI < kRowGroups; gI++) {
+      if ((uint32_t)gI < groupsM) {
+#pragma unroll
+        for (int j = gI * kGroupRows; j < (gI + 1) * kGroupRows; j++) {
+          const uint32_t r = min(wave + kWaves * j, wM);
+          const uint32_t rowStart = offOut + (m0 + r) * a.strideOutM;
+          const uint32_t sRow = (outWord - offOut + rowStart) & (LE - 1);
+          const int32_t k = min(max((int32_t)(tk * kTile) - (int32_t)sRow + (int32_t)lane, 0), (int32_t)volMk - 1);
+          // (a window that lies wholly beyond the run's end repeats the run's last element, which
+          // every LDS row from rowLo on holds in that case)
+          v[j] = tile[max(k - kBase, (int32_t)rowLo)][r];
+          dstOff[j] = rowStart + (uint32_t)k;
+        }
+      }
+    }
+#pragma unroll
+    for (int gI = 0; gI < kRowGroups; gI++) {
+      if ((uint32_t)gI < groupsM) {
+#pragma unroll
+        for (int j = gI * kGroupRows; j < (gI + 1) * kGroupRows; j++) stg<NT>(out + dstOff[j], v[j]);
       }
     }
   }
@@ -480,7 +505,7 @@ bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk,
     if ((uint64_t)xcdChunk * kNumXcd < logical) return false;
     blocks = (uint64_t)xcdChunk * kNumXcd;
   }
-  return blocks > 0 && blocks <= 0x7fffffffull;
+  return blocks > 0 && blocks <= 0x7fffffffull && blocks * kTileThreads <= CUTT_HIP_MAX_GRID_LANES;
 }
 
 // Allow dynamic LDS up to the device limit for a kernel (once per process and kernel).
@@ -564,8 +589,10 @@ hipError_t launchKernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t 
 extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
-      a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 5 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1))
+      a->tilesM != (a->volMm + kTile - 1) / kTile || (a->alignedStores != 0 && a->alignedStores != 1) ||
+      a->tilesK != (a->volMk + (a->alignedStores ? 128 / a->elemSize - 1 : 0) + kTile - 1) / kTile ||
+      a->order < 0 || a->order > 5 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1) ||
+      (a->alignedStores && a->grouped))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
@@ -582,8 +609,10 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);
 #define CUTT_LAUNCH_TILED(T, NT)                                                                        \
-  return (int)(a->grouped ? launchKernel(tiledKernel<T, NT, true>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
-                          : launchKernel(tiledKernel<T, NT, false>, grid, block, 0, s, *a, (const T*)in, (T*)out))
+  return (int)(a->alignedStores                                                                         \
+                   ? launchKernel(tiledAlignedKernel<T, NT>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
+                   : (a->grouped ? launchKernel(tiledKernel<T, NT, true>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
+                                 : launchKernel(tiledKernel<T, NT, false>, grid, block, 0, s, *a, (const T*)in, (T*)out)))
 #define CUTT_LAUNCH_TILED_NT(T)                                \
   switch (a->cachePolicy) {                                    \
     case 0: CUTT_LAUNCH_TILED(T, 0);                           \
@@ -648,7 +677,7 @@ extern "C" int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int ca
   const uint64_t n16 = bytes / 16;
   const uint32_t tailWords = (uint32_t)((bytes % 16) / 4);
   const uint64_t blocks = std::max<uint64_t>(1, (n16 + kCopyThreads - 1) / kCopyThreads);
-  if (blocks > 0x7fffffffull) return (int)hipErrorInvalidConfiguration;
+  if (blocks > 0x7fffffffull || blocks * kCopyThreads > CUTT_HIP_MAX_GRID_LANES) return (int)hipErrorInvalidConfiguration;
   const dim3 grid((uint32_t)blocks), block(kCopyThreads);
   switch (cachePolicy) {
     case 0: return (int)launchKernel(copyKernel<0>, grid, block, 0, s, (const Vec16*)in, (Vec16*)out, n16, tailWords);
@@ -771,7 +800,7 @@ static uint64_t packedGrid(const cuttHipPackedArgs* a) {
     if ((uint64_t)a->xcdChunk * kNumXcd < blocks) return 0;
     blocks = (uint64_t)a->xcdChunk * kNumXcd;
   }
-  return blocks <= 0x7fffffffull ? blocks : 0;
+  return blocks <= 0x7fffffffull && blocks * (uint64_t)a->numThreads <= CUTT_HIP_MAX_GRID_LANES ? blocks : 0;
 }
 
 extern "C" int cuttHipValidatePacked(const cuttHipPackedArgs* a) {

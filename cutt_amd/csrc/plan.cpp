@@ -451,6 +451,9 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
                              : (pb.elemSize == 8 && plan.ldsBytes >= 10 * 1024) ? 2 : 4;
     a.itemsPerBlock = (int)std::max<int64_t>(1, std::min<int64_t>(maxItems, items / std::max<int64_t>(wanted, 1)));
   }
+  // (workgroups x lanes must fit a 32-bit count: more items per workgroup if they would not)
+  const int64_t maxBlocks = (int64_t)(CUTT_HIP_MAX_GRID_LANES / (uint64_t)a.numThreads) - kNumXcd;
+  if (ceilDiv(items, a.itemsPerBlock) > maxBlocks) a.itemsPerBlock = (int)ceilDiv(items, maxBlocks);
   plan.numBlocks = ceilDiv(items, a.itemsPerBlock);
   if (opt.xcdAware && plan.numBlocks >= 64) {
     a.xcdChunk = (uint32_t)ceilDiv(plan.numBlocks, kNumXcd);
@@ -533,16 +536,17 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.strideInK = (uint32_t)pb.strideIn[rk];
     a.strideOutM = (uint32_t)pb.strideOut[0];
     a.tilesM = (int)tilesM;
-    a.tilesK = (int)ceilDiv(sp.volMk, kTile);
+    a.alignedStores = opt.tiledAligned > 0 ? 1 : 0;
+    a.tilesK = (int)ceilDiv(sp.volMk + (a.alignedStores ? 128 / pb.elemSize - 1 : 0), kTile);
     a.volMbar = (int)sp.volMbar;
     TileOrdering o;
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
                                  sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
-    a.grouped = opt.tiledGrouped > 0 ? 1 : 0;  // -1: decided from the model's estimate later
+    a.grouped = opt.tiledGrouped > 0 && !a.alignedStores ? 1 : 0;  // -1: decided from the model's estimate later
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
-    plan.ldsBytes = (size_t)kTile * (kTile + 1) * pb.elemSize;
+    plan.ldsBytes = (size_t)(kTile + (a.alignedStores ? 128 / pb.elemSize - 1 : 0)) * (kTile + 1) * pb.elemSize;
   } else {
     cuttHipTiledCopyArgs& a = plan.tcopy;
     std::memset(&a, 0, sizeof(a));
@@ -565,7 +569,8 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     plan.ldsBytes = 0;
   }
   plan.numThreads = 256;
-  return plan.numBlocks <= 0x7fffffffll;
+  // one tile per workgroup: a tensor with tens of millions of tiny tiles has no Tiled candidate
+  return plan.numBlocks <= 0x7fffffffll && (uint64_t)plan.numBlocks * 256u <= CUTT_HIP_MAX_GRID_LANES;
 }
 
 bool sameCandidate(const Split& a, const Split& b) {

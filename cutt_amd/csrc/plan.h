@@ -137,6 +137,7 @@ struct PlannerOptions {
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
   int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3-5: strips of 8 tiles along Mm
   bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
+  int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups

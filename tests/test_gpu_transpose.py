@@ -452,6 +452,54 @@ def test_tiled_with_four_rows_per_lane_in_flight(gpu, monkeypatch):
         assert info.method_name == "Tiled" and info.tiledGrouped == want
 
 
+def test_tiled_with_line_aligned_stores(gpu, monkeypatch):
+    # The Tiled kernel's instance in which every tile row stores its own window of 64 elements that
+    # starts on a 128-byte line: forced on shapes whose output runs are shorter than a line, shorter
+    # than a tile, a little longer than a tile, with uniform and with rotating misalignment, both
+    # widths; the last tile along Mk may lie wholly beyond some rows' ends.
+    import torch
+    import cutt_amd as cutt
+    cases = [((43, 67), (1, 0)), ((64, 64), (1, 0)), ((65, 127, 3), (1, 0, 2)), ((130, 9, 70), (2, 1, 0)),
+             ((1000, 30, 777), (2, 1, 0)), ((17, 5, 300), (2, 1, 0)), ((300, 5, 17), (2, 1, 0)),
+             ((129, 3, 257, 31), (2, 1, 0, 3)), ((200, 3), (1, 0)), ((70, 40), (1, 0)), ((96, 2, 66), (2, 1, 0)),
+             ((64, 32, 96), (2, 1, 0)), ((33, 7, 5, 95), (3, 1, 2, 0))]
+    monkeypatch.setenv("CUTT_TILED_ALIGNED", "1")
+    cutt.set_method_override(cutt.METHOD_TILED)
+    try:
+        for dim, perm in cases:
+            for es in (4, 8):
+                say("aligned-store tiled dim=%s perm=%s es=%d" % (dim, perm, es))
+                info = gpu.check_case(list(dim), list(perm), es)
+                assert info.method_name == "Tiled"
+        # an output buffer that itself starts off the line grid
+        dim, perm, es = [130, 9, 70], [2, 1, 0], 4
+        vol = int(np.prod(dim))
+        data = gpu.seeded(vol, es, seed=5)
+        d_in = gpu.to_device(data)
+        big = torch.full((vol + 64,), -1, dtype=d_in.dtype, device="cuda")
+        import oracle
+        for shift in (1, 7, 32, 33):
+            d_out = big[shift:shift + vol]
+            rc, h = cutt.cuttPlan(len(dim), dim, perm, es, gpu.stream_handle())
+            assert rc == cutt.CUTT_SUCCESS
+            big.fill_(-1)
+            gpu.run_plan(h, d_in, d_out)
+            cutt.cuttDestroy(h)
+            assert np.array_equal(gpu.to_host(d_out, es), oracle.transpose(dim, perm, data))
+            assert bool((big[:shift] == -1).all()) and bool((big[shift + vol:] == -1).all())
+    finally:
+        cutt.set_method_override(0)
+
+
+def test_measuring_planner_on_a_tensor_with_millions_of_tiny_tiles(gpu):
+    # 50 million 2 x 2 tiles would need a grid beyond the dispatch limit: no such candidate may
+    # be timed (it would "win" with a truncated grid)
+    info = gpu.check_case([2, 7, 2, 14, 17141, 3], [2, 1, 5, 3, 4, 0], 4, how="measure")
+    assert info.numBlocks * info.numThreads < 2 ** 32
+    info = gpu.check_case([2, 7, 2, 14, 171412, 3], [2, 1, 5, 3, 4, 0], 4, how="measure")
+    assert info.numBlocks * info.numThreads < 2 ** 32
+
+
 def test_every_candidate_of_random_midsize_tensors(gpu):
     # Seeded random tensors of 0.3-2 M elements, ranks 3-7: every candidate of the enumeration runs
     # on the GPU (all elements-per-lane, cache-policy and offset-width instances the planner can

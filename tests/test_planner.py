@@ -121,6 +121,18 @@ def test_two_to_the_31_elements_and_more(cutt):
     assert infos and all(i.volMbar < 2 ** 31 for i in infos)
 
 
+def test_no_grid_beyond_the_dispatch_limit(cutt):
+    # workgroups x lanes of a launch must fit a 32-bit count (the runtime truncates a larger grid
+    # without an error): a Tiled candidate with tens of millions of 2 x 2 tiles is not offered, and
+    # packed candidates take more work items per workgroup instead
+    for dim, perm, es in [((2, 7, 2, 14, 171412, 3), (2, 1, 5, 3, 4, 0), 4), ((2, 3, 2, 2, 4000000, 2), (2, 1, 0, 5, 4, 3), 8),
+                          ((3, 2, 16000000, 2), (1, 0, 3, 2), 4)]:
+        infos, best = method_set(cutt, dim, perm, es)
+        assert infos
+        for i in infos:
+            assert i.numBlocks * i.numThreads < 2 ** 32, (dim, perm, i.as_dict())
+
+
 def test_invalid_problems_rejected(cutt):
     for dim, perm, es in [((4, 4), (0, 0), 4), ((4, 1), (1, 0), 4), ((4, 4), (1, 0), 2), ((4,), (0,), 4),
                           ((4, 4), (1, 2), 8), ((65536, 65536), (1, 0), 4)]:
