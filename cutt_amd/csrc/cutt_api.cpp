@@ -80,7 +80,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(dim[i]);
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
-                           "CUTT_MAX_ITEMS", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
+                           "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
                            "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
@@ -383,6 +383,7 @@ PlannerOptions plannerOptions(int forceMethod) {
     if (v == 1 || v == 2 || v == 4 || v == 8 || v == 16) opt.elemsPerThread = v;
   }
   if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_ITEM_ORDER")) opt.itemOrder = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("CUTT_CACHE_POLICY")) {
     const int v = std::atoi(e);
@@ -911,7 +912,7 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
     case 2:
       if (!packed) return -1;
       v = {p.packed.numThreads, p.packed.volMbar, p.packed.itemsPerBlock, p.packed.padShift,
-           p.packed.ldsElems, p.packed.xcdChunk, p.packed.elemsPerThread};
+           p.packed.ldsElems, p.packed.xcdChunk, p.packed.elemsPerThread, p.packed.itemOrder};
       for (int i = 0; i < 2; i++) {
         const cuttHipSplitRank& sr = p.packed.split[i];
         v.insert(v.end(), {sr.numSplit, sr.slabFloor, sr.slabRem, sr.strideIn, sr.strideOut});

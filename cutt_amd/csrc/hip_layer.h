@@ -173,9 +173,15 @@ typedef struct cuttHipSplitRank {
  * Packed and PackedSplit methods.  A staged block is the index set Mmk with up to two of its
  * ranks cut into slabs (typically the last rank of the input-contiguous set and the last rank of
  * the output-contiguous set, which makes the block a 2-D tile over fused rank sets).  Work items
- * are (Mbar position m, slab s1, slab s0), numbered w = (m*numSplit1 + s1)*numSplit0 + s0;
- * workgroup b handles items [b*itemsPerBlock, (b+1)*itemsPerBlock).  The slab sizes select the
- * table class: cls[(s0 < slabRem0) + 2*(s1 < slabRem1)].  Packed is the case without split ranks.
+ * are (Mbar position m, slab s1, slab s0); workgroup b handles the items numbered
+ * [b*itemsPerBlock, (b+1)*itemsPerBlock).  Two numberings (itemOrder):
+ *   0: w = (m*numSplit1 + s1)*numSplit0 + s0 - a workgroup walks neighbouring slabs;
+ *   1: w = ((mb*numSplit1 + s1)*numSplit0 + s0)*itemsPerBlock + mi with m = mb*itemsPerBlock + mi
+ *      (numbers whose m >= volMbar are skipped) - a workgroup keeps its slabs and walks
+ *      itemsPerBlock Mbar positions, neighbouring workgroups have neighbouring slabs.
+ * The slab sizes select the table class: cls[(s0 < slabRem0) + 2*(s1 < slabRem1)]; a workgroup that
+ * meets another class reloads its lanes' table entries (a round trip to memory), which order 1
+ * never does.  Packed is the case without split ranks.
  */
 typedef struct cuttHipPackedArgs {
   int elemSize;
@@ -183,6 +189,7 @@ typedef struct cuttHipPackedArgs {
   int volMbar;
   cuttHipSplitRank split[2];
   int itemsPerBlock;
+  int itemOrder;       /* numbering of the work items, see above */
   int elemsPerThread;  /* 1, 2, 4, 8 or (4-byte elements only) 16: numThreads*elemsPerThread >= vol of every class */
   int padShift;        /* LDS slot(p) = p + (p >> padShift); 31 = no padding */
   int ldsElems;        /* element slots in the LDS data buffer (padding included) */
@@ -197,6 +204,11 @@ typedef struct cuttHipPackedArgs {
   cuttHipMbar mbar;
 } cuttHipPackedArgs;
 
+/* Work-item numbers of these arguments (some of them empty in order 1), or -1 if beyond 31 bits. */
+long long cuttHipPackedItemNumbers(const cuttHipPackedArgs* args);
+/* Work-item number w -> Mbar position, slab indices and table class, as the kernel computes them;
+ * returns 0 if the number is empty (order 1, m beyond volMbar). */
+int cuttHipDecodeItem(const cuttHipPackedArgs* args, uint32_t w, uint32_t* m, uint32_t* s0, uint32_t* s1, int* cls);
 /* Bytes of LDS the packed kernel needs for these arguments. */
 size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a);
 /* Vector registers per lane of the packed kernel instance for this element size, elements per lane

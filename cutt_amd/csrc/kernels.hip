@@ -338,13 +338,16 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   const uint32_t tid = threadIdx.x;
   const uint32_t nt = blockDim.x;
   const uint32_t ns0 = a.split[0].numSplit, ns1 = a.split[1].numSplit;
-  const uint32_t totalItems = (uint32_t)a.volMbar * ns0 * ns1;
+  const uint32_t ipb = (uint32_t)a.itemsPerBlock;
+  const bool byMbar = a.itemOrder == 1;  // the workgroup keeps its slabs and walks Mbar positions
+  const uint32_t totalItems = byMbar ? (((uint32_t)a.volMbar + ipb - 1) / ipb) * ns0 * ns1 * ipb
+                                     : (uint32_t)a.volMbar * ns0 * ns1;
   // XCD-aware numbering: XCD x (= blockIdx.x % 8) walks its own contiguous chunk of the work
   // items, so that neighbouring slabs and Mbar positions share an L2.
   uint32_t lb = blockIdx.x;
   if (a.xcdChunk) lb = (blockIdx.x % kNumXcd) * (uint32_t)a.xcdChunk + blockIdx.x / kNumXcd;
-  const uint32_t w0 = lb * (uint32_t)a.itemsPerBlock;
-  const uint32_t w1 = min(w0 + (uint32_t)a.itemsPerBlock, totalItems);
+  const uint32_t w0 = lb * ipb;
+  uint32_t w1 = min(w0 + ipb, totalItems);
   const uint32_t rem0 = a.split[0].slabRem, rem1 = a.split[1].slabRem;
   const int padShift = a.padShift;
 
@@ -359,10 +362,12 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
 
   // Work item w -> slab class and the item's base offsets (all wave-uniform).
   auto locate = [&](uint32_t w, int& c, uint32_t& offIn, uint32_t& offOut) __attribute__((always_inline)) {
-    const uint32_t t = fastDivide(w, div0.mul, div0.shift, div0.add);
-    const uint32_t s0 = w - t * ns0;
-    const uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
+    const uint32_t slab = byMbar ? lb : w;
+    const uint32_t t = fastDivide(slab, div0.mul, div0.shift, div0.add);
+    const uint32_t s0 = slab - t * ns0;
+    uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
     const uint32_t s1 = t - m * ns1;
+    if (byMbar) m = m * ipb + (w - w0);
     c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
     const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
     const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
@@ -443,6 +448,12 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // gather and the stores of item w, so they overlap, and the wait for them (the memory counter
   // counts loads and stores in issue order) does not also wait for those stores to complete.
   if (w0 >= w1) return;
+  if (byMbar) {
+    // the numbers of this workgroup whose Mbar position lies beyond the rank's end are empty
+    const uint32_t mFirst = fastDivide(fastDivide(lb, div0.mul, div0.shift, div0.add), div1.mul, div1.shift, div1.add) * ipb;
+    if (mFirst >= (uint32_t)a.volMbar) return;
+    w1 = min(w1, w0 + ((uint32_t)a.volMbar - mFirst));
+  }
   uint32_t w = w0, offIn, offOut;
   int cls;
   locate(w, cls, offIn, offOut);
@@ -790,12 +801,9 @@ extern "C" int cuttHipPreparePacked(void) {
 
 // Number of workgroups of a packed launch (0 = the work items do not fit a grid).
 static uint64_t packedGrid(const cuttHipPackedArgs* a) {
-  uint64_t items = (uint64_t)a->volMbar;
-  for (int i = 0; i < 2; i++) {
-    items *= (uint64_t)std::max(1, a->split[i].numSplit);
-    if (items > 0x7fffffffull) return 0;
-  }
-  uint64_t blocks = (items + a->itemsPerBlock - 1) / a->itemsPerBlock;
+  const long long items = cuttHipPackedItemNumbers(a);
+  if (items < 1) return 0;
+  uint64_t blocks = ((uint64_t)items + a->itemsPerBlock - 1) / a->itemsPerBlock;
   if (a->xcdChunk) {
     if ((uint64_t)a->xcdChunk * kNumXcd < blocks) return 0;
     blocks = (uint64_t)a->xcdChunk * kNumXcd;
@@ -807,6 +815,7 @@ extern "C" int cuttHipValidatePacked(const cuttHipPackedArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
       (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
+      (a->itemOrder != 0 && a->itemOrder != 1) ||
       (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
        a->elemsPerThread != 8 && !(a->elemsPerThread == 16 && a->elemSize == 4)) ||
       (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) ||

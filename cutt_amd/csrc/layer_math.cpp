@@ -43,6 +43,33 @@ extern "C" int cuttHipFinishMbar(cuttHipMbar* mb) {
   return 0;
 }
 
+extern "C" long long cuttHipPackedItemNumbers(const cuttHipPackedArgs* a) {
+  const unsigned long long slabs = (unsigned long long)a->split[0].numSplit * (unsigned long long)a->split[1].numSplit;
+  unsigned long long n = (unsigned long long)a->volMbar * slabs;
+  if (a->itemOrder == 1) {
+    const unsigned long long ipb = (unsigned long long)a->itemsPerBlock;
+    n = (((unsigned long long)a->volMbar + ipb - 1) / ipb) * slabs * ipb;
+  }
+  return n > 0x7fffffffull ? -1 : (long long)n;
+}
+
+extern "C" int cuttHipDecodeItem(const cuttHipPackedArgs* a, uint32_t w, uint32_t* m, uint32_t* s0, uint32_t* s1, int* cls) {
+  const uint32_t ns0 = (uint32_t)a->split[0].numSplit, ns1 = (uint32_t)a->split[1].numSplit;
+  uint32_t slab = w, mi = 0, ipb = 1;
+  if (a->itemOrder == 1) {
+    ipb = (uint32_t)a->itemsPerBlock;
+    slab = w / ipb;
+    mi = w - slab * ipb;
+  }
+  const uint32_t t = cuttHipDivide(slab, a->split[0].div);
+  *s0 = slab - t * ns0;
+  const uint32_t mb = cuttHipDivide(t, a->split[1].div);
+  *s1 = t - mb * ns1;
+  *m = mb * ipb + mi;
+  *cls = (*s0 < (uint32_t)a->split[0].slabRem ? 1 : 0) + (*s1 < (uint32_t)a->split[1].slabRem ? 2 : 0);
+  return *m < (uint32_t)a->volMbar;
+}
+
 extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) {
   const size_t b = (size_t)a->ldsElems * a->elemSize;
   return (b + 15) & ~(size_t)15;

@@ -261,12 +261,17 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const cuttHipPackedArgs& a = plan.packed;
     const uint32_t ns0 = (uint32_t)a.split[0].numSplit, ns1 = (uint32_t)a.split[1].numSplit;
     const uint32_t items = (uint32_t)a.volMbar * ns0 * ns1;
-    const int ns = (numSamples == 0 || (uint32_t)numSamples > items) ? (int)items : numSamples;
-    std::uniform_int_distribution<uint32_t> pick(0, items - 1);
-    for (int i = 0; i < ns; i++) {
-      const uint32_t w = ((uint32_t)ns == items) ? (uint32_t)i : pick(rng);
-      const uint32_t s0 = w % ns0, t = w / ns0, s1 = t % ns1, m = t / ns1;
-      const int cls = (s0 < (uint32_t)a.split[0].slabRem ? 1 : 0) + (s1 < (uint32_t)a.split[1].slabRem ? 2 : 0);
+    const uint32_t numbers = (uint32_t)cuttHipPackedItemNumbers(&a);  // some are empty in item order 1
+    const bool all = numSamples == 0 || (uint32_t)numSamples > items;
+    const int ns = all ? (int)items : numSamples;
+    std::uniform_int_distribution<uint32_t> pick(0, numbers - 1);
+    int taken = 0;
+    for (uint32_t i = 0; all ? i < numbers : taken < ns; i++) {
+      const uint32_t w = all ? i : pick(rng);
+      uint32_t s0, s1, m;
+      int cls;
+      if (!cuttHipDecodeItem(&a, w, &m, &s0, &s1, &cls)) continue;
+      taken++;
       const int64_t p0 = (int64_t)s0 * a.split[0].slabFloor + std::min<int64_t>(s0, a.split[0].slabRem);
       const int64_t p1 = (int64_t)s1 * a.split[1].slabFloor + std::min<int64_t>(s1, a.split[1].slabRem);
       int64_t offIn, offOut;

@@ -141,6 +141,8 @@ struct PlannerOptions {
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
+  int itemOrder = -1;        // Packed/PackedSplit work-item numbering: -1 = planner's choice, 0 = a workgroup walks
+                             // neighbouring slabs, 1 = it keeps its slabs and walks Mbar positions
   int maxItemsPerBlock = 0;  // Packed/PackedSplit: work items one workgroup handles at most; 0 = by item size
   int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores
   int mbarOrder = 2;        // order of the Mbar ranks: 0 = input order, 1 = output order,

@@ -136,7 +136,9 @@ int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
  *   what 1: tile geometry: volMm, volMk, strideInK, strideOut(M or K), tilesM, tilesK, volMbar, order,
  *           xcdChunk, superM, superK
  *   what 2: packed scalars: numThreads, volMbar, itemsPerBlock, padShift, ldsElems, xcdChunk,
- *           elemsPerThread, then for each of the two split slots: numSplit, slabFloor, slabRem,
+ *           elemsPerThread, itemOrder (0: work item w = (m*numSplit1 + s1)*numSplit0 + s0; 1: a
+ *           workgroup keeps its slabs, w = ((mb*numSplit1 + s1)*numSplit0 + s0)*itemsPerBlock + mi,
+ *           m = mb*itemsPerBlock + mi), then for each of the two split slots: numSplit, slabFloor, slabRem,
  *           strideIn, strideOut
  *   what 3: class scalars: vol, inCont, outCont
  *   what 4: rowIn[] (vol/inCont input offsets, one per contiguous run)

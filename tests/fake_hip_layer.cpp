@@ -59,5 +59,28 @@ int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs*, const void*, void*, void
 int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void*, void*, void*) { touch(a); return 0; }
 int cuttHipLaunchCopy(const void*, void*, size_t, int, void*) { return 0; }
 int cuttHipPreparePacked(void) { return 0; }
+int cuttHipScratch(void** ptr, size_t* bytes) {
+  static unsigned char scratch[CUTT_HIP_SCRATCH_BYTES];
+  *ptr = scratch;
+  *bytes = sizeof(scratch);
+  return 0;
+}
+int cuttHipLaunchTableBuild(const cuttHipTableBuildArgs* a, void*) {
+  auto radix = [](const cuttHipRadixList& l, uint32_t i) {
+    uint32_t off = 0;
+    for (int k = 0; k < l.n; k++) {
+      off += (i % l.extent[k]) * l.stride[k];
+      i /= l.extent[k];
+    }
+    return off;
+  };
+  for (uint32_t i = 0; i < a->count[0]; i++) a->rowIn[i] = radix(a->list[0], i);
+  for (uint32_t i = 0; i < a->count[1]; i++) a->rowOut[i] = radix(a->list[1], i);
+  for (uint32_t i = 0; i < a->count[2]; i++) {
+    const uint32_t pos = radix(a->list[2], i);
+    a->shIdx[i] = (uint16_t)(pos + (pos >> a->padShift));
+  }
+  return 0;
+}
 int cuttHipPackedRegsPerLaneLoaded(int, int, int) { return -1; }
 }

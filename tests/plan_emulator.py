@@ -105,15 +105,17 @@ def emulate(cands, idx, data):
 
     # Packed / PackedSplit
     sc = [int(v) for v in cands.data(idx, 2)]
-    num_threads, vol_mbar, items_per_block, pad_shift, lds_elems, xcd_chunk, elems_per_thread = sc[:7]
-    splits = [sc[7:12], sc[12:17]]  # numSplit, slabFloor, slabRem, strideIn, strideOut
+    num_threads, vol_mbar, items_per_block, pad_shift, lds_elems, xcd_chunk, elems_per_thread, item_order = sc[:8]
+    splits = [sc[8:13], sc[13:18]]  # numSplit, slabFloor, slabRem, strideIn, strideOut
     assert num_threads % 64 == 0 and 64 <= num_threads <= 1024
     # 16 elements per lane exist for 4-byte elements only
     assert elems_per_thread in (1, 2, 4, 8) or (elems_per_thread == 16 and data.dtype.itemsize == 4)
     off_in, off_out = _mbar_offsets(mbar, vol_mbar)
     ns0, ns1 = splits[0][0], splits[1][0]
     total_items = vol_mbar * ns0 * ns1
-    logical_blocks = -(-total_items // items_per_block)
+    assert item_order in (0, 1)
+    numbers = total_items if item_order == 0 else -(-vol_mbar // items_per_block) * ns0 * ns1 * items_per_block
+    logical_blocks = -(-numbers // items_per_block)
     if xcd_chunk:
         # workgroup b handles logical block (b % 8) * xcd_chunk + b // 8: every logical block once
         assert info.numBlocks == 8 * xcd_chunk and 8 * xcd_chunk >= logical_blocks
@@ -145,13 +147,24 @@ def emulate(cands, idx, data):
         src_p = which[sh]
         assert src_p.min() >= 0, "gather reads an LDS slot that was never written"
         classes[c] = (in_off[src_p], out_off)
-    for w in range(total_items):
-        t, s0 = divmod(w, ns0)
-        m, s1 = divmod(t, ns1)
+    seen = 0
+    for w in range(numbers):
+        if item_order == 0:
+            t, s0 = divmod(w, ns0)
+            m, s1 = divmod(t, ns1)
+        else:  # the workgroup keeps its slabs and walks items_per_block Mbar positions
+            slab, mi = divmod(w, items_per_block)
+            t, s0 = divmod(slab, ns0)
+            mb, s1 = divmod(t, ns1)
+            m = mb * items_per_block + mi
+            if m >= vol_mbar:
+                continue
+        seen += 1
         c = (1 if s0 < splits[0][2] else 0) + (2 if s1 < splits[1][2] else 0)
         p0 = s0 * splits[0][1] + min(s0, splits[0][2])
         p1 = s1 * splits[1][1] + min(s1, splits[1][2])
         src_rel, dst_rel = classes[c]
         scatter(off_out[m] + p0 * splits[0][4] + p1 * splits[1][4] + dst_rel,
                 off_in[m] + p0 * splits[0][3] + p1 * splits[1][3] + src_rel)
+    assert seen == total_items
     return out, count
