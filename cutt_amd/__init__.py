@@ -9,8 +9,8 @@ from .api import (  # noqa: F401
     CUTT_SUCCESS, CUTT_INVALID_PLAN, CUTT_INVALID_PARAMETER, CUTT_INVALID_DEVICE,
     CUTT_INTERNAL_ERROR, CUTT_UNDEFINED_ERROR,
     METHOD_NAMES, METHOD_TRIVIAL, METHOD_PACKED, METHOD_PACKEDSPLIT, METHOD_TILED, METHOD_TILEDCOPY,
-    CuttError, PlanInfo, lib, lib_path,
+    CuttError, PlanInfo, StreamCounts, lib, lib_path,
     cuttPlan, cuttPlanMeasure, cuttPlanFromCandidate, cuttExecute, cuttExecuteNoAlloc, cuttDestroy,
-    get_plan_info, set_method_override, clear_plan_cache, get_last_measurement, reduce_ranks, Candidates,
+    get_plan_info, count_address_stream, set_method_override, clear_plan_cache, get_last_measurement, reduce_ranks, Candidates,
 )
 from .build import build  # noqa: F401

@@ -64,6 +64,16 @@ class PlanInfo(ctypes.Structure):
         return d
 
 
+class StreamCounts(ctypes.Structure):
+    """Mirror of struct cuttStreamCounts (include/cutt_ext.h)."""
+    _fields_ = [(n, ctypes.c_double) for n in ("rdInstr", "wrInstr", "rdInstrIdle", "wrInstrIdle", "rdLines", "wrLines",
+                                               "rdSectors", "wrSectors", "wrPartialLines", "ldsCycles")] + \
+               [("ldsMaxDegree", ctypes.c_int)]
+
+    def as_dict(self):
+        return {name: getattr(self, name) for name, _ in self._fields_}
+
+
 _HERE = os.path.dirname(os.path.abspath(__file__))
 _lib = None
 
@@ -99,6 +109,9 @@ def lib():
     l.cuttDestroy.restype = ctypes.c_int
     l.cuttGetPlanInfo.argtypes = [ctypes.c_uint, ctypes.POINTER(PlanInfo)]
     l.cuttGetPlanInfo.restype = ctypes.c_int
+    l.cuttCountAddressStream.argtypes = [ctypes.c_uint, ctypes.c_int, ctypes.POINTER(StreamCounts),
+                                         ctypes.POINTER(StreamCounts)]
+    l.cuttCountAddressStream.restype = ctypes.c_int
     l.cuttSetMethodOverride.argtypes = [ctypes.c_int]
     l.cuttSetMethodOverride.restype = None
     l.cuttGetMethodOverride.argtypes = []
@@ -189,6 +202,15 @@ def get_plan_info(handle):
     if rc != CUTT_SUCCESS:
         raise CuttError(rc, "cuttGetPlanInfo")
     return info
+
+
+def count_address_stream(handle, num_samples=0):
+    """(counts on the device, counts by the host model) for the plan's address stream."""
+    dev, mod = StreamCounts(), StreamCounts()
+    rc = lib().cuttCountAddressStream(ctypes.c_uint(handle), int(num_samples), ctypes.byref(dev), ctypes.byref(mod))
+    if rc != CUTT_SUCCESS:
+        raise CuttError(rc, "cuttCountAddressStream")
+    return dev, mod
 
 
 def set_method_override(method):

@@ -800,6 +800,43 @@ extern "C" cuttResult cuttGetPlanInfo(cuttHandle handle, cuttPlanInfo* info) {
   return CUTT_SUCCESS;
 }
 
+extern "C" cuttResult cuttCountAddressStream(cuttHandle handle, int numSamples, cuttStreamCounts* onDevice,
+                                             cuttStreamCounts* byModel) {
+  if (!onDevice || !byModel || numSamples < 0) return CUTT_INVALID_PARAMETER;
+  std::shared_ptr<StoredPlan> sp;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    auto it = gPlans.find(handle);
+    if (it == gPlans.end()) return CUTT_INVALID_PLAN;
+    sp = it->second;
+  }
+  Plan& p = sp->plan;
+  if (p.method == kTrivial) return CUTT_INVALID_PARAMETER;
+  try {
+    cuttHipStreamCounts d;
+    std::memset(&d, 0, sizeof(d));
+    int rc;
+    if (p.method == kTiled) rc = cuttHipCountTiled(&p.tiled, &d, p.stream);
+    else if (p.method == kTiledCopy) rc = cuttHipCountTiledCopy(&p.tcopy, &d, p.stream);
+    else rc = cuttHipCountPacked(&p.packed, &d, p.stream);
+    if (rc != 0) return CUTT_INTERNAL_ERROR;
+    *onDevice = cuttStreamCounts{(double)d.rdInstr, (double)d.wrInstr, (double)d.rdInstrIdle, (double)d.wrInstrIdle,
+                                 (double)d.rdLines, (double)d.wrLines, (double)d.rdSectors, (double)d.wrSectors,
+                                 (double)d.wrPartialLines, (double)d.ldsCycles, (int)d.ldsMaxDegree};
+    // the host model's walk over a copy of the plan (the plan itself keeps its estimate)
+    Plan q = p.clone();
+    int deviceID;
+    cuttHipDeviceProps props;
+    if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+    if (!estimatePlan(q, props, numSamples)) return CUTT_INTERNAL_ERROR;
+    *byModel = cuttStreamCounts{q.model.rdInstr, q.model.wrInstr, 0.0, 0.0, q.model.rdLines, q.model.wrLines,
+                                q.model.rdSectors, q.model.wrSectors, q.model.wrPartialLines, q.model.ldsCycles, 0};
+  } catch (...) {
+    return CUTT_INTERNAL_ERROR;
+  }
+  return CUTT_SUCCESS;
+}
+
 extern "C" void cuttSetMethodOverride(int method) {
   std::lock_guard<std::mutex> lock(gMutex);
   gMethodOverride = (method > 0 && method < kNumMethods) ? method : 0;

@@ -277,6 +277,24 @@ int cuttHipLaunchTableBuild(const cuttHipTableBuildArgs* args, void* stream);
 #define CUTT_HIP_SCRATCH_BYTES (1u << 20)
 int cuttHipScratch(void** ptr, size_t* bytes);
 
+/*
+ * What the address stream of a plan's kernel amounts to, counted on the device by kernels that
+ * replay it (count_kernels.hip): wavefront-level load and store instructions that carry data, those
+ * whose lanes all repeat an edge element ("idle"), distinct 128-byte lines and 32-byte sectors per
+ * instruction summed over the launch, partly written lines at the ends of the output runs, LDS
+ * cycles of the packed kernel's gathers, and the largest LDS bank-conflict degree met.
+ */
+typedef struct cuttHipStreamCounts {
+  unsigned long long rdInstr, wrInstr, rdInstrIdle, wrInstrIdle;
+  unsigned long long rdLines, wrLines, rdSectors, wrSectors, wrPartialLines, ldsCycles;
+  unsigned int ldsMaxDegree;
+} cuttHipStreamCounts;
+
+/* Launch the counting kernel for these (validated) arguments on `stream`, wait, return the totals. */
+int cuttHipCountTiled(const cuttHipTiledArgs* args, cuttHipStreamCounts* out, void* stream);
+int cuttHipCountTiledCopy(const cuttHipTiledCopyArgs* args, cuttHipStreamCounts* out, void* stream);
+int cuttHipCountPacked(const cuttHipPackedArgs* args, cuttHipStreamCounts* out, void* stream);
+
 /* Plain copy of `bytes` bytes (a multiple of 4) for the Trivial method; cachePolicy as above. */
 int cuttHipLaunchCopy(const void* in, void* out, size_t bytes, int cachePolicy, void* stream);
 /* One-time kernel attribute setup of the packed kernels on the current device (idempotent). */

@@ -174,13 +174,14 @@ Counts packedSample(const Plan& p, int cls, int64_t offIn, int64_t offOut) {
   const int es = p.pb.elemSize;
   const PackedTables& t = p.tab[cls];
   Counts c;
-  std::vector<int64_t> lines;
+  std::vector<int64_t> lines, sectors;  // distinct 128-byte lines / 32-byte sectors of one request
   lines.reserve(128);
+  sectors.reserve(256);
   // Reads: wavefront requests cover 64 consecutive input-compact positions.
   for (int p0 = 0; p0 < t.vol; p0 += 64) {
     const int p1 = std::min(t.vol, p0 + 64);
     lines.clear();
-    double sectors = 0;
+    sectors.clear();
     int q = p0;
     while (q < p1) {
       const int row = q / t.inCont, col = q % t.inCont;
@@ -188,12 +189,13 @@ Counts packedSample(const Plan& p, int cls, int64_t offIn, int64_t offOut) {
       const int64_t pos = offIn + t.rowIn[row] + col;
       const int64_t b0 = pos * es, b1 = (pos + n) * es;
       for (int64_t l = b0 / kLineBytes; l <= (b1 - 1) / kLineBytes; l++) lines.push_back(l);
-      sectors += (double)((b1 - 1) / kSectorBytes - b0 / kSectorBytes + 1);
+      for (int64_t l = b0 / kSectorBytes; l <= (b1 - 1) / kSectorBytes; l++) sectors.push_back(l);
       q += n;
     }
     std::sort(lines.begin(), lines.end());
     c.rdLines += (double)(std::unique(lines.begin(), lines.end()) - lines.begin());
-    c.rdSectors += sectors;
+    std::sort(sectors.begin(), sectors.end());
+    c.rdSectors += (double)(std::unique(sectors.begin(), sectors.end()) - sectors.begin());
     c.rdInstr += 1;
   }
   // Writes: 64 consecutive output-compact positions per request.
@@ -201,7 +203,7 @@ Counts packedSample(const Plan& p, int cls, int64_t offIn, int64_t offOut) {
   for (int q0 = 0; q0 < t.vol; q0 += 64) {
     const int q1 = std::min(t.vol, q0 + 64);
     lines.clear();
-    double sectors = 0;
+    sectors.clear();
     int q = q0;
     while (q < q1) {
       const int row = q / t.outCont, col = q % t.outCont;
@@ -209,12 +211,13 @@ Counts packedSample(const Plan& p, int cls, int64_t offIn, int64_t offOut) {
       const int64_t pos = offOut + t.rowOut[row] + col;
       const int64_t b0 = pos * es, b1 = (pos + n) * es;
       for (int64_t l = b0 / kLineBytes; l <= (b1 - 1) / kLineBytes; l++) lines.push_back(l);
-      sectors += (double)((b1 - 1) / kSectorBytes - b0 / kSectorBytes + 1);
+      for (int64_t l = b0 / kSectorBytes; l <= (b1 - 1) / kSectorBytes; l++) sectors.push_back(l);
       q += n;
     }
     std::sort(lines.begin(), lines.end());
     c.wrLines += (double)(std::unique(lines.begin(), lines.end()) - lines.begin());
-    c.wrSectors += sectors;
+    std::sort(sectors.begin(), sectors.end());
+    c.wrSectors += (double)(std::unique(sectors.begin(), sectors.end()) - sectors.begin());
     c.wrInstr += 1;
     // LDS gather: conflict degree over 4-byte banks; 8-byte words occupy two banks.
     std::fill(bank.begin(), bank.end(), 0);

@@ -147,6 +147,33 @@ int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
 long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                              long long maxCount);
 
+/* ---- the address stream of a plan, counted on the device ------------------
+ *
+ * Kernels that take a plan's launch arguments and replay the transpose kernel's address stream
+ * (same workgroup numbering, same index arithmetic, same tables, no data moved) count, with 64-lane
+ * ballots, what the cost model counts on the host; the call also returns the host model's walk of
+ * the same plan over numSamples sampled work items (0 = every work item, then the two must agree
+ * exactly).  Counterpart of the reference's cuttGpuModelKernel (src/cuttGpuModelKernel.cu:686-782),
+ * which its library never calls; here a GPU test does.
+ *
+ *   instructions: wavefront-wide loads / stores that carry data; "idle" ones only repeat an edge
+ *   element (the kernels clamp indices instead of branching; the host model does not count them)
+ *   lines, sectors: distinct 128-byte / 32-byte blocks per instruction, summed
+ *   wrPartialLines: ends of output runs that do not fall on a line boundary
+ *   ldsCycles: Packed/PackedSplit, per gather instruction conflict degree * words + words
+ *   ldsMaxDegree (device only): largest bank-conflict degree met (Tiled: of the padded tile)
+ */
+typedef struct cuttStreamCounts {
+  double rdInstr, wrInstr, rdInstrIdle, wrInstrIdle;
+  double rdLines, wrLines, rdSectors, wrSectors, wrPartialLines, ldsCycles;
+  int ldsMaxDegree;
+} cuttStreamCounts;
+
+/* CUTT_INVALID_PLAN for an unknown handle, CUTT_INVALID_PARAMETER for a Trivial plan (a copy has
+ * no index arithmetic to check) or null pointers.  Synchronises the plan's stream. */
+cuttResult cuttCountAddressStream(cuttHandle handle, int numSamples, cuttStreamCounts* onDevice,
+                                  cuttStreamCounts* byModel);
+
 /* ---- counters of the cost model (known-answer tests) --------------------- */
 int cuttModelGlTransactionsSeg(const int* seg, int n);
 int cuttModelGlTransactionsCont(int pos, int n, int accWidth);

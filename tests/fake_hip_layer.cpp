@@ -59,6 +59,9 @@ int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs*, const void*, void*, void
 int cuttHipLaunchPacked(const cuttHipPackedArgs* a, const void*, void*, void*) { touch(a); return 0; }
 int cuttHipLaunchCopy(const void*, void*, size_t, int, void*) { return 0; }
 int cuttHipPreparePacked(void) { return 0; }
+int cuttHipCountTiled(const cuttHipTiledArgs*, cuttHipStreamCounts*, void*) { return 1; }
+int cuttHipCountTiledCopy(const cuttHipTiledCopyArgs*, cuttHipStreamCounts*, void*) { return 1; }
+int cuttHipCountPacked(const cuttHipPackedArgs*, cuttHipStreamCounts*, void*) { return 1; }
 int cuttHipScratch(void** ptr, size_t* bytes) {
   static unsigned char scratch[CUTT_HIP_SCRATCH_BYTES];
   *ptr = scratch;
