@@ -14,9 +14,9 @@ ROCM_LIB = "/opt/rocm/lib"
 
 
 def hip_objects():
-    objs = [os.path.join(CSRC, n) for n in ("hip_layer.o", "kernels.o")]
+    objs = [os.path.join(CSRC, n) for n in ("hip_layer.o", "kernels.o", "count_kernels.o")]
     if not all(os.path.exists(o) for o in objs):
-        subprocess.check_call(["make", "-s", "-C", CSRC, "hip_layer.o", "kernels.o"])
+        subprocess.check_call(["make", "-s", "-C", CSRC, "hip_layer.o", "kernels.o", "count_kernels.o"])
     return objs
 
 
