@@ -177,6 +177,33 @@ def test_random_ranks_up_to_15(gpu):
             gpu.check_case(dim, perm, es)
 
 
+def test_highest_ranks(gpu):
+    # Every extent is at least 2 and a tensor has fewer than 2^32 elements, so rank 31 is the highest
+    # rank that exists; the per-rank tables hold 32.  Ranks 20-28 against the oracle (all extents 2,
+    # a few 3), random and reversing permutations, every method the planner offers.
+    import cutt_amd as cutt
+    rng = np.random.default_rng(31)
+    for rank in (20, 24, 26, 28):
+        dim = [2] * rank
+        if rank <= 24:
+            for i in rng.choice(rank, size=2, replace=False):
+                dim[int(i)] = 3
+        for perm in ([int(p) for p in rng.permutation(rank)], list(range(rank - 1, -1, -1))):
+            es = 4 if rank >= 26 else 8
+            for method in (0, cutt.METHOD_TILED, cutt.METHOD_PACKED, cutt.METHOD_PACKEDSPLIT):
+                cutt.set_method_override(method)
+                try:
+                    rc, h = cutt.cuttPlan(rank, dim, perm, es, gpu.stream_handle())
+                    if rc != cutt.CUTT_SUCCESS:
+                        assert method != 0
+                        continue
+                    cutt.cuttDestroy(h)
+                    say("rank %d perm=%s es=%d method %d" % (rank, perm, es, method))
+                    info = gpu.check_case(dim, perm, es)
+                finally:
+                    cutt.set_method_override(0)
+
+
 def test_ten_streams(gpu):
     # reference test4: ten plans on ten streams executing into the same buffers
     import torch

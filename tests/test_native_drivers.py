@@ -92,6 +92,21 @@ def test_cutt_bench_random_suites_short(planner):
 
 
 @pytest.mark.gpu
+def test_rank_31_the_highest_rank_that_exists():
+    # 31 extents of 2 = 2^31 four-byte elements (8.6 GB per buffer), random permutation; checked on
+    # the device by closed form.  A rank-32 tensor would have 2^32 elements, beyond the API's limit.
+    import os
+    import numpy as np
+    exe = os.path.join(BIN, "cutt_bench")
+    perm = [str(int(p)) for p in np.random.default_rng(5).permutation(31)]
+    for extra in ([], ["-measure"]):
+        r = subprocess.run([exe, "-elemsize", "4", "-bufelems", "2147483648", "-dim"] + ["2"] * 31 + ["-permutation"] + perm +
+                           ["-nomemcpy"] + extra, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+        assert r.returncode == 0, r.stdout[-2000:]
+        assert "bench OK" in r.stdout
+
+
+@pytest.mark.gpu
 def test_tensor_above_4GB_uses_wide_offsets():
     # 671 088 640 doubles = 5.4 GB per buffer: byte offsets no longer fit 32 bits
     import os
