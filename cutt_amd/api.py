@@ -52,6 +52,7 @@ class PlanInfo(ctypes.Structure):
         ("cachePolicy", ctypes.c_int), ("elemsPerThread", ctypes.c_int),
         ("rdEdgeDist", ctypes.c_double), ("wrEdgeDist", ctypes.c_double),
         ("tiledGrouped", ctypes.c_int), ("superM", ctypes.c_int), ("superK", ctypes.c_int),
+        ("tiledAligned", ctypes.c_int), ("itemOrder", ctypes.c_int),
     ]
 
     @property

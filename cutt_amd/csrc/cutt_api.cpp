@@ -80,7 +80,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(dim[i]);
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
-                           "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
+                           "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
                            "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
@@ -201,6 +201,8 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
                                       : (p.method == kTiledCopy ? p.tcopy.cachePolicy : p.packed.cachePolicy);
   o.elemsPerThread = p.packed.elemsPerThread;
   o.tiledGrouped = p.method == kTiled ? p.tiled.grouped : 0;
+  o.tiledAligned = p.method == kTiled ? p.tiled.alignedStores : 0;
+  o.itemOrder = (p.method == kPacked || p.method == kPackedSplit) ? p.packed.itemOrder : 0;
   o.superM = p.method == kTiled ? (int)p.tiled.superM : (p.method == kTiledCopy ? (int)p.tcopy.superM : 0);
   o.superK = p.method == kTiled ? (int)p.tiled.superK : (p.method == kTiledCopy ? (int)p.tcopy.superK : 0);
   o.rdEdgeDist = p.model.rdEdgeDist;
@@ -383,6 +385,7 @@ PlannerOptions plannerOptions(int forceMethod) {
     if (v == 1 || v == 2 || v == 4 || v == 8 || v == 16) opt.elemsPerThread = v;
   }
   if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
+  if (const char* e = std::getenv("CUTT_PAD_SHIFT")) opt.padShift = std::min(31, std::max(1, std::atoi(e)));
   if (const char* e = std::getenv("CUTT_ITEM_ORDER")) opt.itemOrder = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("CUTT_CACHE_POLICY")) {
@@ -614,7 +617,10 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
     } else {
       cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
     }
-    if (plans[best].method == kTiled) cur.tiledGrouped = plans[best].tiled.grouped;
+    if (plans[best].method == kTiled) {
+      cur.tiledGrouped = plans[best].tiled.grouped;
+      cur.tiledAligned = plans[best].tiled.alignedStores;
+    }
     const PlannerOptions start = cur;
 
     // Tries `v`; keeps it (and returns true) if it is faster than the best so far.
@@ -654,6 +660,16 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
       if (!failed && plans[best].method == kTiled && !std::getenv("CUTT_TILED_GROUPED")) {
         PlannerOptions v = cur;
         v.tiledGrouped = 1 - cur.tiledGrouped;
+        if (tryVariant(v, false)) cur = v;
+      }
+      // every tile row storing its own line-aligned window (measured: +2...+4 % on some 8-byte
+      // tensors with output runs off the 128-byte grid, -5...-15 % on others, so only by trial)
+      if (!failed && plans[best].method == kTiled && !std::getenv("CUTT_TILED_ALIGNED") &&
+          ((int64_t)plans[best].tiled.volMk * plans[best].pb.elemSize % 128 != 0 ||
+           (int64_t)plans[best].tiled.strideOutM * plans[best].pb.elemSize % 128 != 0)) {
+        PlannerOptions v = cur;
+        v.tiledAligned = 1;
+        v.tiledGrouped = 0;
         if (tryVariant(v, false)) cur = v;
       }
     } else {

@@ -25,7 +25,7 @@ constexpr int64_t kNumXcd = 8;          // XCDs (private L2s); workgroup b runs 
 
 inline int64_t ceilDiv(int64_t a, int64_t b) { return (a + b - 1) / b; }
 inline int roundUp64(int64_t v) { return (int)(ceilDiv(v, 64) * 64); }
-inline int64_t paddedSlots(int64_t vol) { return vol ? (vol - 1) + ((vol - 1) >> kPadShift) + 1 : 0; }
+inline int64_t paddedSlots(int64_t vol, int shift = kPadShift) { return vol ? (vol - 1) + ((vol - 1) >> shift) + 1 : 0; }
 }  // namespace
 
 const char* methodName(int method) {
@@ -391,7 +391,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   std::memset(&a, 0, sizeof(a));
   a.elemSize = pb.elemSize;
   a.volMbar = (int)sp.volMbar;
-  a.padShift = kPadShift;
+  a.padShift = opt.padShift > 0 ? opt.padShift : kPadShift;
   a.cachePolicy = opt.cachePolicy;
   a.volume = pb.volume;
   a.wideOffsets = (opt.wideOffsets || (uint64_t)pb.volume * (uint64_t)pb.elemSize > (1ull << 32)) ? 1 : 0;
@@ -422,7 +422,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
     k.outDiv = cuttHipMakeDivisor((uint32_t)oc);
     a.maxVol = std::max(a.maxVol, k.vol);
   }
-  const int64_t slots = paddedSlots(a.maxVol);
+  const int64_t slots = paddedSlots(a.maxVol, a.padShift);
   if (slots > kMaxLdsSlots) return false;
   a.ldsElems = (int)slots;
   plan.ldsBytes = cuttHipPackedLdsBytes(&a);

@@ -56,6 +56,9 @@ typedef struct cuttPlanInfo {
   double rdEdgeDist, wrEdgeDist;
   int tiledGrouped;     /* Tiled: 1 if a lane keeps 4 instead of 16 tile rows in flight */
   int superM, superK;   /* Tiled/TiledCopy: shape of the super-tiles the workgroups walk (tiled orders 3-5) */
+  int tiledAligned;     /* Tiled: 1 if every tile row stores its own line-aligned window of its output run */
+  int itemOrder;        /* Packed/PackedSplit: 0 = a workgroup walks neighbouring slabs, 1 = it keeps its slabs
+                           and walks Mbar positions */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */
