@@ -439,7 +439,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // more tiles along Mm 0.97 times.
     if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0 && bytes > cacheBytes) factor *= 1.1;  // measured at 1.9-3.7 GB
   } else {
-    factor = 1.05 + (es == 4 ? 0.17 : 0.093) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
+    factor = 1.05 + (es == 4 ? 0.17 : 0.15) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +
              0.10 * (rdAmp - 1.0) * far(r.rdEdgeDist);
     // Residuals of all candidates in reach of the best one over 600 random tensors and the 80
@@ -447,7 +447,13 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // model's own ratios): what the estimate lacked is the cost of lines that are touched twice
     // when the workgroup with the neighbouring run comes late - the whole excess of lines, not
     // only the partly written ones - and a bump for output runs of 64 bytes to 1 KB.
-    factor += 0.30 * (wrAmp - 1.0) * far(r.wrEdgeDist) + (es == 4 ? 0.08 : 0.10) * (rdAmp - 1.0) * far(r.rdEdgeDist);
+    // The excess counts lines per request; what a late neighbour can cost is bounded by the lines
+    // that two workgroups share (a 4000-byte output run written by 512-byte requests has an excess
+    // of 0.21 but shares 0.05 of its lines: (200000,2,500) -> (500,2,200000) with 8-byte elements,
+    // cut along the first rank, measured 611-633 us with such runs and 732 us with 64-byte input
+    // runs read twice, which the uncapped term ranked the other way round).
+    factor += 0.30 * std::min(wrAmp - 1.0, 2.0 * partial) * far(r.wrEdgeDist) +
+              (es == 4 ? 0.08 : 0.10) * (rdAmp - 1.0) * far(r.rdEdgeDist);
     {
       const double outBytes = (double)plan.split.volMmkOutCont * es;
       if (outBytes >= 64.0 && outBytes <= 1024.0) factor *= es == 4 ? 1.07 : 1.03;
