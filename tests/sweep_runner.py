@@ -7,6 +7,7 @@ Every output is checked on the device: the input holds each element's linear ind
 expectation is torch's own permute + contiguous of that index tensor (an independent routine).
 Shared by tests/test_gpu_c5_sweep.py and bench.py --sweep."""
 import ctypes
+import os
 import time
 
 import numpy as np
@@ -69,12 +70,22 @@ def run_tensor(cfg, reps=4, planners=("plan", "measure"), log=None):
     for how in planners:
         if log:
             log("%s %s dim=%s perm=%s es=%d" % (res["name"], how, dim, perm, es))
-        t0 = time.perf_counter()
-        if how == "measure":
-            rc, h = cutt.cuttPlanMeasure(len(dim), dim, perm, es, st, d_in.data_ptr(), d_out.data_ptr())
-        else:
-            rc, h = cutt.cuttPlan(len(dim), dim, perm, es, st)
-        plan_ms = (time.perf_counter() - t0) * 1e3
+        # plan-creation time is that of a first call: the library's cache of decisions is switched
+        # off for the call (an earlier test of the same process may have planned this tensor)
+        saved = os.environ.get("CUTT_PLAN_CACHE")
+        os.environ["CUTT_PLAN_CACHE"] = "0"
+        try:
+            t0 = time.perf_counter()
+            if how == "measure":
+                rc, h = cutt.cuttPlanMeasure(len(dim), dim, perm, es, st, d_in.data_ptr(), d_out.data_ptr())
+            else:
+                rc, h = cutt.cuttPlan(len(dim), dim, perm, es, st)
+            plan_ms = (time.perf_counter() - t0) * 1e3
+        finally:
+            if saved is None:
+                del os.environ["CUTT_PLAN_CACHE"]
+            else:
+                os.environ["CUTT_PLAN_CACHE"] = saved
         assert rc == cutt.CUTT_SUCCESS, (rc, cfg, how)
         info = cutt.get_plan_info(h)
 
