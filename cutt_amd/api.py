@@ -53,6 +53,7 @@ class PlanInfo(ctypes.Structure):
         ("rdEdgeDist", ctypes.c_double), ("wrEdgeDist", ctypes.c_double),
         ("tiledGrouped", ctypes.c_int), ("superM", ctypes.c_int), ("superK", ctypes.c_int),
         ("tiledAligned", ctypes.c_int), ("itemOrder", ctypes.c_int),
+        ("numPieces", ctypes.c_int), ("numShapes", ctypes.c_int),
     ]
 
     @property
@@ -127,6 +128,11 @@ def lib():
     l.cuttCandidatesCreate.restype = vp
     l.cuttCandidatesCreateEx.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t, ctypes.c_size_t]
     l.cuttCandidatesCreateEx.restype = vp
+    llp = ctypes.POINTER(ctypes.c_longlong)
+    l.cuttCandidatesCreateStrided.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t, llp, llp, ctypes.c_size_t]
+    l.cuttCandidatesCreateStrided.restype = vp
+    l.cuttSlabDecomposition.argtypes = [ctypes.c_int, ip, ip, ctypes.c_size_t, ctypes.c_longlong, llp, ctypes.c_longlong]
+    l.cuttSlabDecomposition.restype = ctypes.c_longlong
     l.cuttCandidatesFree.argtypes = [vp]
     l.cuttCandidatesFree.restype = None
     l.cuttCandidatesCount.argtypes = [vp]
@@ -239,12 +245,40 @@ def reduce_ranks(dim, permutation):
     return list(rd[:k]), list(rp[:k])
 
 
+def slab_decomposition(dim, permutation, sizeofType, span_limit=0):
+    """How the library cuts a tensor into pieces one launch can address: (shapes, pieces) with
+    shapes = [dict(dim, perm, stride_in, stride_out)] and pieces = [(shape, base_in, base_out)];
+    None if it cannot be cut."""
+    n = lib().cuttSlabDecomposition(len(dim), _ints(dim), _ints(permutation), int(sizeofType), int(span_limit), None, 0)
+    if n < 0:
+        return None
+    buf = (ctypes.c_longlong * n)()
+    lib().cuttSlabDecomposition(len(dim), _ints(dim), _ints(permutation), int(sizeofType), int(span_limit), buf, n)
+    v = [int(x) for x in buf]
+    num_shapes, num_pieces = v[0], v[1]
+    pos = 2
+    shapes = []
+    for _ in range(num_shapes):
+        r = v[pos]
+        pos += 1
+        f = [v[pos + i * r: pos + (i + 1) * r] for i in range(4)]
+        pos += 4 * r
+        shapes.append(dict(dim=f[0], perm=f[1], stride_in=f[2], stride_out=f[3]))
+    pieces = [tuple(v[pos + 3 * i: pos + 3 * i + 3]) for i in range(num_pieces)]
+    return shapes, pieces
+
+
 class Candidates:
     """The planner's candidate list for a problem, built for MI355X properties without a GPU."""
 
-    def __init__(self, dim, permutation, sizeofType, lds_per_block=0):
-        self._l = lib().cuttCandidatesCreateEx(len(dim), _ints(dim), _ints(permutation), int(sizeofType),
-                                               int(lds_per_block))
+    def __init__(self, dim, permutation, sizeofType, lds_per_block=0, stride_in=None, stride_out=None):
+        if stride_in is None:
+            self._l = lib().cuttCandidatesCreateEx(len(dim), _ints(dim), _ints(permutation), int(sizeofType),
+                                                   int(lds_per_block))
+        else:  # one piece of a larger tensor, with that tensor's element strides
+            lls = lambda v: (ctypes.c_longlong * len(v))(*[int(x) for x in v])
+            self._l = lib().cuttCandidatesCreateStrided(len(dim), _ints(dim), _ints(permutation), int(sizeofType),
+                                                        lls(stride_in), lls(stride_out), int(lds_per_block))
         if not self._l:
             raise ValueError("invalid transpose problem")
 

@@ -29,6 +29,7 @@
 #include "hip_layer.h"
 #include "model.h"
 #include "plan.h"
+#include "slab.h"
 
 using namespace cutt;
 
@@ -36,6 +37,10 @@ namespace {
 
 struct StoredPlan {
   Plan plan;
+  // A tensor beyond what one launch addresses (slab.h): one launch per piece, with the plan of the
+  // piece's shape - `plan` for shape 0, more[s - 1] for shape s.  Empty for every other tensor.
+  std::vector<Plan> more;
+  std::vector<SlabPiece> pieces;
   int numCandidates = 0;
   double planMs = 0;
   double usMeasured = 0;
@@ -127,19 +132,28 @@ int methodOverrideLocked() {
   return gMethodOverride;
 }
 
-// Same checks as reference src/cutt.cpp:59-82.  The reference's int arithmetic implies fewer than
-// 2^31 elements; here the limit is 2^32 - 1 (element offsets are unsigned 32-bit in the kernels,
-// byte addresses 64-bit).
-cuttResult checkInput(int rank, const int* dim, const int* perm, size_t sizeofType) {
+// Largest rank the API accepts.  One launch handles at most CUTT_MAX_RANK ranks and 2^32 - 1
+// elements (element offsets are unsigned 32-bit in the kernels, byte addresses 64-bit); a tensor
+// beyond either is cut into pieces within those limits (slab.h).
+constexpr int kMaxApiRank = 64;
+constexpr long long kMaxElements = 1ll << 46;
+
+// Same checks as reference src/cutt.cpp:59-82 (whose int arithmetic implies fewer than 2^31
+// elements).  `large` receives whether the tensor has to be cut into pieces; an entry point that
+// passes none refuses such tensors.
+cuttResult checkInput(int rank, const int* dim, const int* perm, size_t sizeofType, bool* large = nullptr) {
   if (sizeofType != 4 && sizeofType != 8) return CUTT_INVALID_PARAMETER;
-  if (rank <= 1 || rank > CUTT_MAX_RANK) return CUTT_INVALID_PARAMETER;
+  if (rank <= 1 || rank > kMaxApiRank) return CUTT_INVALID_PARAMETER;
   if (!dim || !perm) return CUTT_INVALID_PARAMETER;
   long long vol = 1;
   for (int i = 0; i < rank; i++) {
     if (dim[i] <= 1) return CUTT_INVALID_PARAMETER;
     vol *= dim[i];
-    if (vol > 0xffffffffll) return CUTT_INVALID_PARAMETER;
+    if (vol > kMaxElements) return CUTT_INVALID_PARAMETER;
   }
+  const bool cut = rank > CUTT_MAX_RANK || slabNeeded(rank, dim, slabSpanLimit());
+  if (cut && !large) return CUTT_INVALID_PARAMETER;
+  if (large) *large = cut;
   std::vector<char> seen(rank, 0);
   for (int i = 0; i < rank; i++) {
     if (perm[i] < 0 || perm[i] >= rank || seen[perm[i]]) return CUTT_INVALID_PARAMETER;
@@ -203,6 +217,8 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.tiledGrouped = p.method == kTiled ? p.tiled.grouped : 0;
   o.tiledAligned = p.method == kTiled ? p.tiled.alignedStores : 0;
   o.itemOrder = (p.method == kPacked || p.method == kPackedSplit) ? p.packed.itemOrder : 0;
+  o.numPieces = 1;
+  o.numShapes = 1;
   o.superM = p.method == kTiled ? (int)p.tiled.superM : (p.method == kTiledCopy ? (int)p.tcopy.superM : 0);
   o.superK = p.method == kTiled ? (int)p.tiled.superK : (p.method == kTiledCopy ? (int)p.tcopy.superK : 0);
   o.rdEdgeDist = p.model.rdEdgeDist;
@@ -401,13 +417,18 @@ PlannerOptions plannerOptions(int forceMethod) {
   return opt;
 }
 
-bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
-               const cuttHipDeviceProps& props, int forceMethod, std::vector<Plan>& plans) {
-  Problem orig, red;
+// The problem as given and with its ranks fused.
+void makeProblems(int rank, const int* dim, const int* perm, size_t sizeofType, Problem& orig, Problem& red) {
   orig.set(rank, dim, perm, (int)sizeofType);
   std::vector<int> redDim, redPerm;
   reduceRanks(rank, dim, perm, redDim, redPerm);
   red.set((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType);
+}
+
+bool enumerate(int rank, const int* dim, const int* perm, size_t sizeofType,
+               const cuttHipDeviceProps& props, int forceMethod, std::vector<Plan>& plans) {
+  Problem orig, red;
+  makeProblems(rank, dim, perm, sizeofType, orig, red);
   return createPlans(orig, red, props, plannerOptions(forceMethod), plans);
 }
 
@@ -420,6 +441,29 @@ cuttResult storePlan(cuttHandle* handle, Plan&& chosen, void* stream, int device
   sp->numCandidates = numCandidates;
   sp->usMeasured = usMeasured;
   if (sp->plan.activate() != 0) return CUTT_INTERNAL_ERROR;
+  sp->planMs = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
+  std::lock_guard<std::mutex> lock(gMutex);
+  *handle = gNextHandle++;
+  if (gPlans.count(*handle)) return CUTT_INTERNAL_ERROR;
+  gPlans.emplace(*handle, std::move(sp));
+  return CUTT_SUCCESS;
+}
+
+// The same for a tensor in pieces: parts[s] is the plan of the pieces of shape s.
+cuttResult storeLargePlan(cuttHandle* handle, std::vector<Plan>&& parts, std::vector<SlabPiece>&& pieces, void* stream,
+                          int deviceID, int numCandidates, double usMeasured,
+                          std::chrono::steady_clock::time_point t0) {
+  std::shared_ptr<StoredPlan> sp = std::make_shared<StoredPlan>();
+  for (Plan& p : parts) {
+    p.stream = stream;
+    p.deviceID = deviceID;
+    if (p.activate() != 0) return CUTT_INTERNAL_ERROR;
+  }
+  sp->plan = std::move(parts[0]);
+  for (size_t s = 1; s < parts.size(); s++) sp->more.push_back(std::move(parts[s]));
+  sp->pieces = std::move(pieces);
+  sp->numCandidates = numCandidates;
+  sp->usMeasured = usMeasured;
   sp->planMs = std::chrono::duration<double, std::milli>(std::chrono::steady_clock::now() - t0).count();
   std::lock_guard<std::mutex> lock(gMutex);
   *handle = gNextHandle++;
@@ -455,12 +499,82 @@ static cuttResult decideHeuristically(int rank, int* dim, int* permutation, size
   return CUTT_SUCCESS;
 }
 
+struct Measured {
+  Plan plan;
+  int numCandidates = 0;
+  double bestUs = 0;
+};
+static cuttResult measureProblem(const Problem& orig, const Problem& red, int force, int deviceID,
+                                 const cuttHipDeviceProps& props, hipStream_t stream, void* idata, void* odata,
+                                 size_t numBytes, Measured& out);
+
+// Elements between the first and the last element of a problem's output, inclusive.
+static int64_t outputSpan(const Problem& pb) {
+  int64_t span = 1;
+  for (int r = 0; r < pb.rank; r++) span += (int64_t)(pb.dim[r] - 1) * pb.strideOut[r];
+  return span;
+}
+
+// cuttPlan / cuttPlanMeasure for a tensor that one launch cannot address: the fused tensor is cut
+// into pieces (slab.h) and every shape of piece is planned like a tensor of its own - by the cost
+// model, or by timing its candidates on the first piece of that shape.
+static cuttResult planLarge(cuttHandle* handle, int rank, int* dim, int* permutation, size_t sizeofType,
+                            hipStream_t stream, bool measure, void* idata, void* odata,
+                            std::chrono::steady_clock::time_point t0) {
+  int deviceID;
+  cuttHipDeviceProps props;
+  if (!currentDevice(deviceID, props)) return CUTT_INTERNAL_ERROR;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  std::vector<int> redDim, redPerm;
+  reduceRanks(rank, dim, permutation, redDim, redPerm);
+  SlabDecomposition dec;
+  if (!slabDecompose((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType, slabSpanLimit(), dec))
+    return CUTT_INVALID_PARAMETER;
+  std::vector<Plan> parts(dec.shapes.size());
+  int numCandidates = 0;
+  double usMeasured = 0;
+  for (size_t s = 0; s < dec.shapes.size(); s++) {
+    const Problem& shape = dec.shapes[s];
+    if (shape.rank > CUTT_MAX_RANK) return CUTT_INVALID_PARAMETER;
+    if (measure) {
+      size_t first = 0;
+      while (dec.pieces[first].shape != (int)s) first++;
+      Measured m;
+      cuttResult r = measureProblem(shape, shape, force, deviceID, props, stream,
+                                    (char*)idata + dec.pieces[first].baseIn * (int64_t)sizeofType,
+                                    (char*)odata + dec.pieces[first].baseOut * (int64_t)sizeofType,
+                                    (size_t)outputSpan(shape) * sizeofType, m);
+      if (r != CUTT_SUCCESS) return r;
+      parts[s] = std::move(m.plan);
+      if (s == 0) { numCandidates = m.numCandidates; usMeasured = m.bestUs; }
+    } else {
+      std::vector<Plan> plans;
+      if (!createPlans(shape, shape, props, plannerOptions(force), plans) || plans.empty()) return CUTT_INTERNAL_ERROR;
+      if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
+      refineMbarOrder(plans, props, force);
+      const int best = chooseHeuristic(plans);
+      if (best < 0) return CUTT_INTERNAL_ERROR;
+      chooseCachePolicy(plans[best], props);
+      if (s == 0) numCandidates = (int)plans.size();
+      parts[s] = std::move(plans[best]);
+    }
+  }
+  return storeLargePlan(handle, std::move(parts), std::move(dec.pieces), (void*)stream, deviceID, numCandidates,
+                        usMeasured, t0);
+}
+
 static cuttResult planImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
                            size_t sizeofType, hipStream_t stream) {
   const auto t0 = std::chrono::steady_clock::now();
   if (!handle) return CUTT_INVALID_PARAMETER;
-  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  bool large = false;
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType, &large);
   if (chk != CUTT_SUCCESS) return chk;
+  if (large) return planLarge(handle, rank, dim, permutation, sizeofType, stream, false, nullptr, nullptr, t0);
 
   int deviceID;
   cuttHipDeviceProps props;
@@ -521,9 +635,11 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
                                   size_t sizeofType, hipStream_t stream, void* idata, void* odata) {
   const auto t0 = std::chrono::steady_clock::now();
   if (!handle) return CUTT_INVALID_PARAMETER;
-  cuttResult chk = checkInput(rank, dim, permutation, sizeofType);
+  bool large = false;
+  cuttResult chk = checkInput(rank, dim, permutation, sizeofType, &large);
   if (chk != CUTT_SUCCESS) return chk;
   if (idata == odata || !idata || !odata) return CUTT_INVALID_PARAMETER;
+  if (large) return planLarge(handle, rank, dim, permutation, sizeofType, stream, true, idata, odata, t0);
 
   int deviceID;
   cuttHipDeviceProps props;
@@ -533,14 +649,24 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
     std::lock_guard<std::mutex> lock(gMutex);
     force = methodOverrideLocked();
   }
+  Problem orig, red;
+  makeProblems(rank, dim, permutation, sizeofType, orig, red);
+  Measured m;
+  chk = measureProblem(orig, red, force, deviceID, props, stream, idata, odata, (size_t)orig.volume * sizeofType, m);
+  if (chk != CUTT_SUCCESS) return chk;
+  return storePlan(handle, std::move(m.plan), (void*)stream, deviceID, m.numCandidates, m.bestUs, t0);
+}
+
+// Times the candidates of one problem on the caller's buffers (`numBytes` of the output are
+// overwritten before every run) and hands back the fastest, activated.
+static cuttResult measureProblem(const Problem& orig, const Problem& red, int force, int deviceID,
+                                 const cuttHipDeviceProps& props, hipStream_t stream, void* idata, void* odata,
+                                 size_t numBytes, Measured& out) {
   std::vector<Plan> plans;
-  if (!enumerate(rank, dim, permutation, sizeofType, props, force, plans)) return CUTT_INTERNAL_ERROR;
+  if (!createPlans(orig, red, props, plannerOptions(force), plans)) return CUTT_INTERNAL_ERROR;
   if (plans.empty()) return CUTT_INTERNAL_ERROR;
   if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
   for (Plan& p : plans) chooseCachePolicy(p, props);
-
-  size_t numBytes = sizeofType;
-  for (int i = 0; i < rank; i++) numBytes *= (size_t)dim[i];
 
   // Candidates the model puts far behind its best are not timed (its error is well inside that
   // margin); CUTT_MEASURE_ALL=1 times every candidate, as the reference does.
@@ -710,7 +836,10 @@ static cuttResult planMeasureImpl(cuttHandle* handle, int rank, int* dim, int* p
       gLastMeasurement[i].numCandidates = (int)plans.size();
     }
   }
-  return storePlan(handle, std::move(plans[best]), (void*)stream, deviceID, (int)plans.size(), bestUs, t0);
+  out.numCandidates = (int)plans.size();
+  out.bestUs = bestUs;
+  out.plan = std::move(plans[best]);
+  return CUTT_SUCCESS;
 }
 
 static cuttResult planFromCandidateImpl(cuttHandle* handle, int rank, int* dim, int* permutation,
@@ -797,7 +926,17 @@ extern "C" cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata) {
   int deviceID;
   if (cuttHipGetDevice(&deviceID) != 0) return CUTT_INTERNAL_ERROR;
   if (deviceID != sp->plan.deviceID) return CUTT_INVALID_DEVICE;
-  if (sp->plan.launch(idata, odata) != 0) return CUTT_INTERNAL_ERROR;
+  if (sp->pieces.empty()) {
+    if (sp->plan.launch(idata, odata) != 0) return CUTT_INTERNAL_ERROR;
+    return CUTT_SUCCESS;
+  }
+  // a tensor in pieces: one launch per piece, all on the plan's stream
+  const int64_t es = sp->plan.pb.elemSize;
+  for (const SlabPiece& piece : sp->pieces) {
+    Plan& p = piece.shape == 0 ? sp->plan : sp->more[piece.shape - 1];
+    if (p.launch((const char*)idata + piece.baseIn * es, (char*)odata + piece.baseOut * es) != 0)
+      return CUTT_INTERNAL_ERROR;
+  }
   return CUTT_SUCCESS;
 }
 
@@ -810,6 +949,10 @@ extern "C" cuttResult cuttGetPlanInfo(cuttHandle handle, cuttPlanInfo* info) {
   auto it = gPlans.find(handle);
   if (it == gPlans.end()) return CUTT_INVALID_PLAN;
   fillInfo(it->second->plan, *info);
+  if (!it->second->pieces.empty()) {
+    info->numPieces = (int)it->second->pieces.size();
+    info->numShapes = 1 + (int)it->second->more.size();
+  }
   info->numCandidates = it->second->numCandidates;
   info->planMs = it->second->planMs;
   info->usMeasured = it->second->usMeasured;
@@ -916,6 +1059,54 @@ extern "C" void* cuttCandidatesCreateEx(int rank, const int* dim, const int* per
   }
   l->best = chooseHeuristic(l->plans);
   return l;
+}
+
+extern "C" void* cuttCandidatesCreateStrided(int rank, const int* dim, const int* permutation, size_t sizeofType,
+                                             const long long* strideIn, const long long* strideOut,
+                                             size_t ldsPerBlock) {
+  if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS || !strideIn || !strideOut) return nullptr;
+  int force;
+  {
+    std::lock_guard<std::mutex> lock(gMutex);
+    force = methodOverrideLocked();
+  }
+  std::vector<int64_t> sIn(strideIn, strideIn + rank), sOut(strideOut, strideOut + rank);
+  Problem pb;
+  if (!pb.setStrided(rank, dim, permutation, (int)sizeofType, sIn.data(), sOut.data())) return nullptr;
+  std::unique_ptr<CandidateList> l(new CandidateList());
+  cuttHipDeviceProps props = defaultMI355XProps();
+  if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
+  if (!createPlans(pb, pb, props, plannerOptions(force), l->plans) || !estimateAll(l->plans, props)) return nullptr;
+  l->best = chooseHeuristic(l->plans);
+  return l.release();
+}
+
+extern "C" long long cuttSlabDecomposition(int rank, const int* dim, const int* permutation, size_t sizeofType,
+                                           long long spanLimit, long long* values, long long maxCount) {
+  bool large = false;
+  if (checkInput(rank, dim, permutation, sizeofType, &large) != CUTT_SUCCESS) return -1;
+  std::vector<int> redDim, redPerm;
+  reduceRanks(rank, dim, permutation, redDim, redPerm);
+  SlabDecomposition dec;
+  if (!slabDecompose((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType,
+                     spanLimit > 0 ? spanLimit : slabSpanLimit(), dec))
+    return -1;
+  std::vector<long long> v = {(long long)dec.shapes.size(), (long long)dec.pieces.size()};
+  for (const Problem& p : dec.shapes) {
+    v.push_back(p.rank);
+    for (int r = 0; r < p.rank; r++) v.push_back(p.dim[r]);
+    for (int r = 0; r < p.rank; r++) v.push_back(p.perm[r]);
+    for (int r = 0; r < p.rank; r++) v.push_back(p.strideIn[r]);
+    for (int r = 0; r < p.rank; r++) v.push_back(p.strideOut[r]);
+  }
+  for (const SlabPiece& q : dec.pieces) {
+    v.push_back(q.shape);
+    v.push_back(q.baseIn);
+    v.push_back(q.baseOut);
+  }
+  if (values)
+    for (long long i = 0; i < std::min<long long>(maxCount, (long long)v.size()); i++) values[i] = v[i];
+  return (long long)v.size();
 }
 
 extern "C" void* cuttCandidatesCreate(int rank, const int* dim, const int* permutation,

@@ -99,6 +99,24 @@ void Problem::set(int rank_, const int* dim_, const int* perm_, int elemSize_) {
     strideOut[perm[j]] = c;
     c *= dim[perm[j]];
   }
+  gapIn.assign(rank, 0);
+  gapOut.assign(rank, 0);
+  dense = true;
+}
+
+bool Problem::setStrided(int rank_, const int* dim_, const int* perm_, int elemSize_, const int64_t* strideIn_,
+                         const int64_t* strideOut_) {
+  set(rank_, dim_, perm_, elemSize_);
+  strideIn.assign(strideIn_, strideIn_ + rank);
+  strideOut.assign(strideOut_, strideOut_ + rank);
+  if (rank < 1 || strideIn[0] != 1 || strideOut[perm[0]] != 1) return false;
+  for (int r = 0; r + 1 < rank; r++) {
+    gapIn[r] = strideIn[r + 1] != strideIn[r] * dim[r];
+    const int a = perm[r], b = perm[r + 1];
+    gapOut[a] = strideOut[b] != strideOut[a] * dim[a];
+    if (gapIn[r] || gapOut[a]) dense = false;
+  }
+  return true;
 }
 
 void reduceRanks(int rank, const int* dim, const int* perm, std::vector<int>& redDim,
@@ -165,6 +183,7 @@ void Split::update(int numMm_, int numMk_, const Problem& pb) {
       break;
     }
     volMmkInCont *= pb.dim[r];
+    if (pb.gapIn[r]) break;
   }
   volMmkOutCont = 1;
   for (int j = 0; j < rank && inMmk[pb.perm[j]]; j++) {
@@ -175,6 +194,7 @@ void Split::update(int numMm_, int numMk_, const Problem& pb) {
       break;
     }
     volMmkOutCont *= pb.dim[r];
+    if (pb.gapOut[r]) break;
   }
 }
 
@@ -336,12 +356,12 @@ void classGeometry(const Split& sp, const Problem& pb, const int* slab, int64_t&
     if (sp.inMmk[r]) v *= blockExtent(sp, pb, r, slab);
   for (int r = 0; r < pb.rank && sp.inMmk[r]; r++) {
     ic *= blockExtent(sp, pb, r, slab);
-    if (sp.splitSlot(r) >= 0) break;
+    if (sp.splitSlot(r) >= 0 || pb.gapIn[r]) break;
   }
   for (int j = 0; j < pb.rank && sp.inMmk[pb.perm[j]]; j++) {
     const int r = pb.perm[j];
     oc *= blockExtent(sp, pb, r, slab);
-    if (sp.splitSlot(r) >= 0) break;
+    if (sp.splitSlot(r) >= 0 || pb.gapOut[r]) break;
   }
   vol = v;
   inCont = ic;
@@ -817,12 +837,16 @@ bool createPlans(const Problem& orig, const Problem& red, const cuttHipDevicePro
                  const PlannerOptions& opt, std::vector<Plan>& plans) {
   bool identity = true;
   for (int i = 0; i < red.rank; i++) identity = identity && red.perm[i] == i;
-  if (identity) {
+  if (identity && red.dense) {
     // Everything fuses into one rank (or would, if the fused extent still fitted an int): a plain
     // copy is the only candidate.
     addTrivial(red, opt, plans);
     return true;
   }
+  // (A piece of a larger tensor whose ranks keep their order is a copy of rows with gaps between
+  // them: the TiledCopy and Packed candidates below handle it.  A single rank with gaps cannot occur:
+  // a strided problem has unit strides in its leading ranks.)
+  if (red.rank < 2) return false;
   addTiled(red, props, opt, plans);
   addPacked(orig, false, props, opt, plans);
   if (red.rank != orig.rank) addPacked(red, true, props, opt, plans);
@@ -857,7 +881,7 @@ static bool classRadixLists(const Plan& plan, int c, std::vector<RadixDim>& rows
     compactIn[r] = cstride;
     cstride *= e;
     if (!inPrefix) rowsIn.push_back({e, pb.strideIn[r]});
-    if (sp.splitSlot(r) >= 0) inPrefix = false;  // ranks after a split rank start new rows
+    if (sp.splitSlot(r) >= 0 || pb.gapIn[r]) inPrefix = false;  // ranks after a split rank or a gap start new rows
   }
   if (cstride != packed.cls[c].vol) return false;
   // Ranks of Mmk in output order.
@@ -871,7 +895,7 @@ static bool classRadixLists(const Plan& plan, int c, std::vector<RadixDim>& rows
     const int e = blockExtent(sp, pb, r, slab);
     gather.push_back({e, compactIn[r]});
     if (!outPrefix) rowsOut.push_back({e, pb.strideOut[r]});
-    if (sp.splitSlot(r) >= 0) outPrefix = false;
+    if (sp.splitSlot(r) >= 0 || pb.gapOut[r]) outPrefix = false;
   }
   return true;
 }

@@ -25,6 +25,9 @@ enum Method { kUnknown = 0, kTrivial = 1, kPacked = 2, kPackedSplit = 3, kTiled 
 const char* methodName(int method);
 
 // A transpose problem: dims (dim[0] fastest), permutation, element size, strides.
+// Usually both tensors are dense (strides follow from the extents).  A piece of a larger tensor
+// (slab.h) keeps the larger tensor's strides: then a rank may not continue where the previous one
+// ends, which gapIn / gapOut record, and only ranks without a gap between them form contiguous runs.
 struct Problem {
   int rank = 0;
   int elemSize = 0;
@@ -33,9 +36,15 @@ struct Problem {
   std::vector<int> inv;        // inv[perm[j]] = j
   std::vector<int64_t> strideIn;   // input stride of input rank r
   std::vector<int64_t> strideOut;  // output stride of input rank r
+  std::vector<char> gapIn;     // gapIn[r]: input rank r+1 does not start where rank r ends
+  std::vector<char> gapOut;    // gapOut[r]: the rank that follows r in the output does not start where r ends
+  bool dense = true;           // no gaps and unit strides of the two leading ranks
   int64_t volume = 0;
 
   void set(int rank, const int* dim, const int* perm, int elemSize);
+  // Same with given strides; false unless the leading rank of each side has stride 1.
+  bool setStrided(int rank, const int* dim, const int* perm, int elemSize, const int64_t* strideIn,
+                  const int64_t* strideOut);
 };
 
 // Fuse runs of ranks that stay adjacent and in order (reference src/cuttplan.cpp:63-126).

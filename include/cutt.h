@@ -54,6 +54,12 @@ typedef enum cuttResult_t {
  *   stream            HIP stream the plan executes on (0 = default stream)
  *
  * The plan is bound to the device that is current at the call.
+ *
+ * Sizes: up to 64 ranks and 2^46 elements.  One kernel launch addresses fewer than 2^32 elements;
+ * a larger tensor (the reference's int volumes end at 2^31 - 1) is cut into pieces, and
+ * cuttExecute issues one launch per piece on the plan's stream.  CUTT_INVALID_PARAMETER beyond
+ * those sizes and for the rare shapes in which the fastest rank of the input lies 2^32 elements
+ * and more apart in the output (or the other way round).
  */
 cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
                     size_t sizeofType, hipStream_t stream);
@@ -95,7 +101,8 @@ cuttResult cuttExecute(cuttHandle handle, void* idata, void* odata);
  * process ends) and launches the same transpose kernel after it on `stream`.  The plan is the
  * one cuttPlan would choose; arguments and checks are those of cuttPlan and cuttExecute.
  *
- * Limits: a plan whose index tables exceed the static memory is refused with
+ * Limits: tensors of 2^32 elements and more are refused (CUTT_INVALID_PARAMETER); a plan whose index
+ * tables exceed the static memory is refused with
  * CUTT_INVALID_PARAMETER and a message on stderr (the tables of the plans this library builds
  * need at most 640 KiB).  Every call on one GPU uses the same static memory: calls on the same
  * stream are ordered and safe, calls whose work may overlap on the GPU (different streams, several

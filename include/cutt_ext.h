@@ -59,6 +59,9 @@ typedef struct cuttPlanInfo {
   int tiledAligned;     /* Tiled: 1 if every tile row stores its own line-aligned window of its output run */
   int itemOrder;        /* Packed/PackedSplit: 0 = a workgroup walks neighbouring slabs, 1 = it keeps its slabs
                            and walks Mbar positions */
+  int numPieces;        /* launches per cuttExecute: 1, or the pieces of a tensor of 2^32 elements and more
+                           (the other fields then describe the plan of the first piece) */
+  int numShapes;        /* different shapes among those pieces (each has a plan of its own): 1..4 */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */
@@ -123,11 +126,29 @@ void* cuttCandidatesCreate(int rank, const int* dim, const int* permutation, siz
  * also produce PackedSplit candidates. */
 void* cuttCandidatesCreateEx(int rank, const int* dim, const int* permutation, size_t sizeofType,
                              size_t ldsPerBlock);
+/* The candidates for one piece of a larger tensor: extents and permutation of the piece, element
+ * strides of the larger tensor (per input rank, for the input and the output side; the leading
+ * rank of each side must have stride 1). */
+void* cuttCandidatesCreateStrided(int rank, const int* dim, const int* permutation, size_t sizeofType,
+                                  const long long* strideIn, const long long* strideOut, size_t ldsPerBlock);
 void cuttCandidatesFree(void* list);
 int cuttCandidatesCount(void* list);
 /* Index of the candidate the cost model ranks best. */
 int cuttCandidatesBest(void* list);
 int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info);
+
+/*
+ * How a tensor is cut into pieces that one launch can address (every piece spans at most
+ * spanLimit elements of the input and of the output; 0 = the library's limit, 2^32 - 1).  The
+ * ranks are fused first.  Copies up to maxCount values into `values` and returns the number
+ * there are, -1 if the tensor cannot be cut (see slab.h):
+ *   numShapes, numPieces,
+ *   per shape: rank, extents[rank], permutation[rank], strideIn[rank], strideOut[rank],
+ *   per piece: shape, baseIn, baseOut (element offsets).
+ * A tensor that needs no cutting comes back as one piece of one shape.
+ */
+long long cuttSlabDecomposition(int rank, const int* dim, const int* permutation, size_t sizeofType,
+                                long long spanLimit, long long* values, long long maxCount);
 
 /*
  * Raw index data of candidate `index`, for checking a plan's address stream

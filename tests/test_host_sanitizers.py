@@ -27,7 +27,7 @@ def hip_objects():
 ])
 def test_planner_under_sanitizer(tmp_path, name, flags, marks):
     exe = str(tmp_path / "planner_stress")
-    srcs = [os.path.join(HERE, "planner_stress.cpp")] + [os.path.join(CSRC, n) for n in ("cutt_api.cpp", "plan.cpp", "model.cpp", "layer_math.cpp")]
+    srcs = [os.path.join(HERE, "planner_stress.cpp")] + [os.path.join(CSRC, n) for n in ("cutt_api.cpp", "plan.cpp", "model.cpp", "layer_math.cpp", "slab.cpp")]
     cmd = (["g++", "-O1", "-g", "-std=c++17", "-pthread"] + flags +
            ["-I" + os.path.join(ROOT, "include"), "-I" + CSRC] + srcs + hip_objects() +
            ["-L" + ROCM_LIB, "-lamdhip64", "-Wl,-rpath," + ROCM_LIB, "-o", exe])
@@ -41,7 +41,7 @@ def test_planner_under_sanitizer(tmp_path, name, flags, marks):
 
 
 FAKE_SRCS = [os.path.join(HERE, n) for n in ("plan_lifetime_stress.cpp", "fake_hip_layer.cpp")] + \
-            [os.path.join(CSRC, n) for n in ("cutt_api.cpp", "plan.cpp", "model.cpp", "layer_math.cpp")]
+            [os.path.join(CSRC, n) for n in ("cutt_api.cpp", "plan.cpp", "model.cpp", "layer_math.cpp", "slab.cpp")]
 
 
 def build_on_fake_layer(exe, flags):
