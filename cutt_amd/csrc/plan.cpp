@@ -538,6 +538,14 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
       if (tilesM >= 16) superM = 4;
     }
   }
+  if (opt.superAuto && (o.order == 5 || o.order == 3) && superM == opt.superM && tilesM > superM && tilesM <= 16) {
+    // A rank of 9..16 tiles is not cut into two strips (5 + 4 ... 8 + 8): one strip as wide as the rank
+    // reads whole input rows.  Forced Tiled plans on 13 random tensors with such a rank (both widths,
+    // with and without Mbar ranks): +2.8 % in the mean, -2 % ... +8 %; the three-rank reversals of the
+    // reference's bench 5 with 13 tiles along Mm and 3 along Mk, (817,1480,148)-like: 749 -> 660 us.
+    // From 17 tiles on a single strip gains nothing in the mean (-7 % ... +9 %) and stays cut.
+    superM = tilesM;
+  }
   int64_t sm = std::min<int64_t>(superM, tilesM), sk = std::min<int64_t>(superK, tilesK);
   // Equal-sized super-tiles: no nearly empty last one (its padding workgroups would leave XCDs idle).
   sm = ceilDiv(tilesM, ceilDiv(tilesM, sm));
