@@ -53,7 +53,7 @@ class PlanInfo(ctypes.Structure):
         ("rdEdgeDist", ctypes.c_double), ("wrEdgeDist", ctypes.c_double),
         ("tiledGrouped", ctypes.c_int), ("superM", ctypes.c_int), ("superK", ctypes.c_int),
         ("tiledAligned", ctypes.c_int), ("itemOrder", ctypes.c_int),
-        ("numPieces", ctypes.c_int), ("numShapes", ctypes.c_int),
+        ("numPieces", ctypes.c_int), ("numShapes", ctypes.c_int), ("wideOffsets", ctypes.c_int),
     ]
 
     @property

@@ -219,6 +219,7 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.itemOrder = (p.method == kPacked || p.method == kPackedSplit) ? p.packed.itemOrder : 0;
   o.numPieces = 1;
   o.numShapes = 1;
+  o.wideOffsets = (p.method == kPacked || p.method == kPackedSplit) ? p.packed.wideOffsets : 0;
   o.superM = p.method == kTiled ? (int)p.tiled.superM : (p.method == kTiledCopy ? (int)p.tcopy.superM : 0);
   o.superK = p.method == kTiled ? (int)p.tiled.superK : (p.method == kTiledCopy ? (int)p.tcopy.superK : 0);
   o.rdEdgeDist = p.model.rdEdgeDist;

@@ -197,7 +197,7 @@ typedef struct cuttHipPackedArgs {
   uint32_t xcdChunk;   /* 0: workgroup b is logical block b; else logical block = (b % 8)*xcdChunk + b/8
                           and the grid has 8*xcdChunk workgroups */
   int cachePolicy;     /* 0 = default, 1 = non-temporal loads, 3 = non-temporal loads and stores */
-  long long volume;    /* elements of the whole tensor (bounds every offset) */
+  long long volume;    /* elements from the first to the last one of the tensor, on its wider side (bounds every offset) */
   int wideOffsets;     /* 0: the tensor is below 4 GB and the kernel keeps 32-bit byte offsets;
                           1: element offsets with 64-bit address arithmetic (required from 4 GB on) */
   cuttHipPackedClass cls[4];

@@ -25,10 +25,10 @@
  *    thousands are in flight: on this chip that streams faster than a
  *    persistent grid-stride loop.
  *
- * All offsets are unsigned 32-bit element offsets (the API limits a tensor to
- * fewer than 2^32 elements; every true offset is below the volume, so the
- * modular sums are exact); the packed kernel turns them into 32-bit byte
- * offsets from a wave-uniform base when the tensor is below 4 GB.
+ * All offsets are unsigned 32-bit element offsets from the pointers of the launch (one launch
+ * spans fewer than 2^32 elements on either side - a larger tensor comes in pieces -; every true
+ * offset is below that span, so the modular sums are exact); the packed kernel turns them into
+ * 32-bit byte offsets from a wave-uniform base when the span is below 4 GB.
  */
 #include <hip/hip_runtime.h>
 

@@ -102,6 +102,7 @@ void Problem::set(int rank_, const int* dim_, const int* perm_, int elemSize_) {
   gapIn.assign(rank, 0);
   gapOut.assign(rank, 0);
   dense = true;
+  span = volume;
 }
 
 bool Problem::setStrided(int rank_, const int* dim_, const int* perm_, int elemSize_, const int64_t* strideIn_,
@@ -116,6 +117,12 @@ bool Problem::setStrided(int rank_, const int* dim_, const int* perm_, int elemS
     gapOut[a] = strideOut[b] != strideOut[a] * dim[a];
     if (gapIn[r] || gapOut[a]) dense = false;
   }
+  int64_t spanIn = 1, spanOut = 1;
+  for (int r = 0; r < rank; r++) {
+    spanIn += (int64_t)(dim[r] - 1) * strideIn[r];
+    spanOut += (int64_t)(dim[r] - 1) * strideOut[r];
+  }
+  span = std::max(spanIn, spanOut);
   return true;
 }
 
@@ -413,8 +420,9 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
   a.volMbar = (int)sp.volMbar;
   a.padShift = opt.padShift > 0 ? opt.padShift : kPadShift;
   a.cachePolicy = opt.cachePolicy;
-  a.volume = pb.volume;
-  a.wideOffsets = (opt.wideOffsets || (uint64_t)pb.volume * (uint64_t)pb.elemSize > (1ull << 32)) ? 1 : 0;
+  // what bounds the offsets is the span: a piece of a larger tensor reaches further than its volume
+  a.volume = pb.span;
+  a.wideOffsets = (opt.wideOffsets || (uint64_t)pb.span * (uint64_t)pb.elemSize > (1ull << 32)) ? 1 : 0;
   for (int i = 0; i < 2; i++) {
     cuttHipSplitRank& sr = a.split[i];
     sr.numSplit = 1;

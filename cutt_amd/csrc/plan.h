@@ -40,6 +40,7 @@ struct Problem {
   std::vector<char> gapOut;    // gapOut[r]: the rank that follows r in the output does not start where r ends
   bool dense = true;           // no gaps and unit strides of the two leading ranks
   int64_t volume = 0;
+  int64_t span = 0;            // elements from the first to the last one, on the wider side (= volume when dense)
 
   void set(int rank, const int* dim, const int* perm, int elemSize);
   // Same with given strides; false unless the leading rank of each side has stride 1.

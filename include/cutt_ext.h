@@ -62,6 +62,8 @@ typedef struct cuttPlanInfo {
   int numPieces;        /* launches per cuttExecute: 1, or the pieces of a tensor of 2^32 elements and more
                            (the other fields then describe the plan of the first piece) */
   int numShapes;        /* different shapes among those pieces (each has a plan of its own): 1..4 */
+  int wideOffsets;      /* Packed/PackedSplit: 1 if the kernel instance does 64-bit address arithmetic (the
+                           tensor, or the piece of a larger one, spans 4 GB and more) */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */

@@ -3,7 +3,7 @@
 A tensor of 2^32 elements and more (or of more than 32 ranks) is beyond the kernels' 32-bit element
 offsets; the library cuts it into pieces and launches one kernel per piece.  Small tensors go
 through the same code when CUTT_SPAN_LIMIT lowers the limit, and are compared with the CPU oracle;
-tensors of 4.3e9 and 8.6e9 elements are checked on the device against a closed form, chunk by chunk,
+tensors of 4.3e9 to 1.7e10 elements are checked on the device against a closed form, chunk by chunk,
 with a value pattern that does not repeat every 2^32 elements (so a base offset that lost its high
 bits cannot pass).
 """
@@ -169,21 +169,27 @@ def test_more_than_2_to_the_32_elements(cutt, dim, perm, es, how):
     assert count_wrong(b, dim, perm, words) == 0
 
 
-def test_rank_33(cutt):
-    """33 ranks of extent 2 (8.6e9 four-byte elements, 34 GB per buffer): the first 29 ranks reversed,
-    the last four swapped in pairs."""
-    dim = [2] * 33
-    perm = list(range(28, -1, -1)) + [30, 29, 32, 31]
-    vol = 2 ** 33
+def test_rank_34(cutt):
+    """34 ranks of extent 2 (1.7e10 four-byte elements, 69 GB per buffer).  The permutation leaves pieces
+    of 2^29 elements (2 GB) that reach 2^31 elements (8 GB) from their base on both sides: the kernel
+    instance with 64-bit addresses has to be chosen by reach, not by volume."""
+    dim = [2] * 34
+    perm = [30, 29, 28, 27, 26, 25, 24, 23, 22, 21, 19, 18, 17, 16, 15, 14, 13, 12, 9, 8, 7, 6, 5, 4, 3, 2, 1, 0,
+            31, 32, 33, 20, 10, 11]
+    vol = 2 ** 34
     a = fill_pattern(vol, 1)
     b = torch.full((vol,), -1, dtype=torch.int32, device="cuda")
-    rc, h = cutt.cuttPlan(33, dim, perm, 4, stream())
+    print("planning", flush=True)
+    rc, h = cutt.cuttPlan(34, dim, perm, 4, stream())
     assert rc == cutt.CUTT_SUCCESS
     info = cutt.get_plan_info(h)
-    print("pieces", info.numPieces, "shapes", info.numShapes, info.method_name, flush=True)
+    print("pieces", info.numPieces, "shapes", info.numShapes, info.method_name, "wide", info.wideOffsets, flush=True)
+    assert info.numPieces == 32
+    assert info.method_name not in ("Packed", "PackedSplit") or info.wideOffsets == 1
     assert cutt.cuttExecute(h, a.data_ptr(), b.data_ptr()) == cutt.CUTT_SUCCESS
     torch.cuda.synchronize()
     assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
+    print("checking", flush=True)
     assert count_wrong(b, dim, perm, 1) == 0
     # ranks beyond 64, and shapes whose leading ranks cannot stay contiguous inside 32-bit offsets, are refused
     assert cutt.cuttPlan(65, [2] * 65, list(range(64, -1, -1)), 4, stream())[0] == cutt.CUTT_INVALID_PARAMETER

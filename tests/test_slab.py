@@ -144,3 +144,14 @@ def test_every_candidate_of_every_piece_shape(cutt, oracle_mod, es):
                     strided += any(a * d != b for a, d, b in zip(s["stride_in"], s["dim"], s["stride_in"][1:]))
     assert checked > 300 and strided > 100
     assert {"Tiled", "TiledCopy", "Packed", "PackedSplit"} <= methods
+
+
+def test_a_small_piece_that_reaches_far_gets_64_bit_addresses(cutt):
+    """The packed kernel keeps 32-bit byte offsets only while everything it can reach lies within
+    4 GB of its base pointers; for a piece of a larger tensor that is its span, not its volume."""
+    far = dict(stride_in=[1, 64, 2 ** 24], stride_out=[2 ** 26, 64, 1])   # 16 x 8 x 16 elements that reach 8 GB
+    near = dict(stride_in=[1, 64, 2 ** 12], stride_out=[2 ** 13, 64, 1])
+    for strides, wide in ((far, 1), (near, 0)):
+        with cutt.Candidates([16, 8, 16], [2, 1, 0], 8, **strides) as c:
+            packed = [c.info(i) for i in range(len(c)) if c.info(i).method_name in ("Packed", "PackedSplit")]
+            assert packed and all(i.wideOffsets == wide for i in packed)
