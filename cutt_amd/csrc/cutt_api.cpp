@@ -403,7 +403,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   }
   if (const char* e = std::getenv("CUTT_PACKED_ROUNDS")) opt.packedRounds = std::max(0, std::atoi(e));
   if (const char* e = std::getenv("CUTT_PAD_SHIFT")) opt.padShift = std::min(31, std::max(1, std::atoi(e)));
-  if (const char* e = std::getenv("CUTT_ITEM_ORDER")) opt.itemOrder = std::atoi(e) != 0 ? 1 : 0;
+  if (const char* e = std::getenv("CUTT_ITEM_ORDER")) opt.itemOrder = std::min(2, std::max(0, std::atoi(e)));
   if (const char* e = std::getenv("CUTT_MAX_ITEMS")) opt.maxItemsPerBlock = std::max(1, std::atoi(e));
   if (const char* e = std::getenv("CUTT_CACHE_POLICY")) {
     const int v = std::atoi(e);

@@ -179,9 +179,14 @@ typedef struct cuttHipSplitRank {
  *   1: w = ((mb*numSplit1 + s1)*numSplit0 + s0)*itemsPerBlock + mi with m = mb*itemsPerBlock + mi
  *      (numbers whose m >= volMbar are skipped) - a workgroup keeps its slabs and walks
  *      itemsPerBlock Mbar positions, neighbouring workgroups have neighbouring slabs.
+ *   2: numbered as in 0, handed out differently: the workgroups of one XCD (of the whole grid when
+ *      xcdChunk is 0) take the numbers of their chunk in turn - the workgroup with index q inside
+ *      a chunk of B workgroups handles chunkStart + q, chunkStart + q + B, ... - so that the items
+ *      in flight at one time are neighbours in memory and a workgroup's next item lies one round
+ *      ahead.
  * The slab sizes select the table class: cls[(s0 < slabRem0) + 2*(s1 < slabRem1)]; a workgroup that
  * meets another class reloads its lanes' table entries (a round trip to memory), which order 1
- * never does.  Packed is the case without split ranks.
+ * never does (and order 2 does most often, when slabs of different sizes exist).  Packed is the case without split ranks.
  */
 typedef struct cuttHipPackedArgs {
   int elemSize;

@@ -346,8 +346,21 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // items, so that neighbouring slabs and Mbar positions share an L2.
   uint32_t lb = blockIdx.x;
   if (a.xcdChunk) lb = (blockIdx.x % kNumXcd) * (uint32_t)a.xcdChunk + blockIdx.x / kNumXcd;
-  const uint32_t w0 = lb * ipb;
-  uint32_t w1 = min(w0 + ipb, totalItems);
+  // The workgroup's items are the numbers wBase + i * wStride, i < count.  Orders 0 and 1: ipb
+  // consecutive numbers.  Order 2: the workgroups of one XCD take the numbers of their chunk in
+  // turn, so that the items in flight at one time are neighbours and a workgroup's next item lies
+  // a whole round ahead.
+  uint32_t wBase = lb * ipb, wStride = 1;
+  uint32_t count = wBase < totalItems ? min(ipb, totalItems - wBase) : 0;
+  if (a.itemOrder == 2) {
+    const uint32_t chunkBlocks = a.xcdChunk ? (uint32_t)a.xcdChunk : gridDim.x;
+    const uint32_t x = lb / chunkBlocks;
+    const uint32_t chunkStart = x * chunkBlocks * ipb;
+    const uint32_t chunkEnd = min(chunkStart + chunkBlocks * ipb, totalItems);
+    wBase = chunkStart + (lb - x * chunkBlocks);
+    wStride = chunkBlocks;
+    count = wBase < chunkEnd ? (chunkEnd - wBase + wStride - 1) / wStride : 0;
+  }
   const uint32_t rem0 = a.split[0].slabRem, rem1 = a.split[1].slabRem;
   const int padShift = a.padShift;
 
@@ -360,14 +373,14 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   const MbarLane mbarLane = loadMbarLane(a.mbar, tid & 63);
   const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
 
-  // Work item w -> slab class and the item's base offsets (all wave-uniform).
-  auto locate = [&](uint32_t w, int& c, uint32_t& offIn, uint32_t& offOut) __attribute__((always_inline)) {
-    const uint32_t slab = byMbar ? lb : w;
+  // The workgroup's i-th item -> slab class and the item's base offsets (all wave-uniform).
+  auto locate = [&](uint32_t i, int& c, uint32_t& offIn, uint32_t& offOut) __attribute__((always_inline)) {
+    const uint32_t slab = byMbar ? lb : wBase + i * wStride;
     const uint32_t t = fastDivide(slab, div0.mul, div0.shift, div0.add);
     const uint32_t s0 = slab - t * ns0;
     uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
     const uint32_t s1 = t - m * ns1;
-    if (byMbar) m = m * ipb + (w - w0);
+    if (byMbar) m = m * ipb + i;
     c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
     const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
     const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
@@ -447,14 +460,14 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // Software pipeline over the workgroup's items: the loads of item w+1 are issued before the LDS
   // gather and the stores of item w, so they overlap, and the wait for them (the memory counter
   // counts loads and stores in issue order) does not also wait for those stores to complete.
-  if (w0 >= w1) return;
+  if (count == 0) return;
   if (byMbar) {
     // the numbers of this workgroup whose Mbar position lies beyond the rank's end are empty
     const uint32_t mFirst = fastDivide(fastDivide(lb, div0.mul, div0.shift, div0.add), div1.mul, div1.shift, div1.add) * ipb;
     if (mFirst >= (uint32_t)a.volMbar) return;
-    w1 = min(w1, w0 + ((uint32_t)a.volMbar - mFirst));
+    count = min(count, (uint32_t)a.volMbar - mFirst);
   }
-  uint32_t w = w0, offIn, offOut;
+  uint32_t w = 0, offIn, offOut;  // index of the item among the workgroup's own
   int cls;
   locate(w, cls, offIn, offOut);
   loadReadSide(cls);
@@ -462,7 +475,7 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   loadWriteSide(cls);  // after the data loads are out: its latency hides behind theirs
   stage();
   for (;;) {
-    if (w + 1 >= w1) {  // last item: nothing to fetch ahead
+    if (w + 1 >= count) {  // last item: nothing to fetch ahead
       __syncthreads();
       gatherAndStore(offOut);
       break;
@@ -815,7 +828,7 @@ extern "C" int cuttHipValidatePacked(const cuttHipPackedArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->numThreads < 64 || a->numThreads > 1024 ||
       (a->numThreads & 63) || a->volMbar < 1 || a->itemsPerBlock < 1 || a->padShift < 1 ||
-      (a->itemOrder != 0 && a->itemOrder != 1) ||
+      a->itemOrder < 0 || a->itemOrder > 2 ||
       (a->elemsPerThread != 1 && a->elemsPerThread != 2 && a->elemsPerThread != 4 &&
        a->elemsPerThread != 8 && !(a->elemsPerThread == 16 && a->elemSize == 4)) ||
       (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) ||

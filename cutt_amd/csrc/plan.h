@@ -152,7 +152,8 @@ struct PlannerOptions {
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16
   int packedRounds = 0;      // > 0: size the grid for this many waves of resident workgroups
   int itemOrder = -1;        // Packed/PackedSplit work-item numbering: -1 = planner's choice, 0 = a workgroup walks
-                             // neighbouring slabs, 1 = it keeps its slabs and walks Mbar positions
+                             // neighbouring slabs, 1 = it keeps its slabs and walks Mbar positions, 2 = the
+                             // workgroups of an XCD take the items of their chunk round by round
   int padShift = 0;          // Packed/PackedSplit: LDS slot(p) = p + (p >> padShift); 0 = the default (5), 31 = no padding
   int maxItemsPerBlock = 0;  // Packed/PackedSplit: work items one workgroup handles at most; 0 = by item size
   int cachePolicy = 1;      // 0 default, 1 non-temporal loads, 3 non-temporal loads and stores

@@ -58,7 +58,8 @@ typedef struct cuttPlanInfo {
   int superM, superK;   /* Tiled/TiledCopy: shape of the super-tiles the workgroups walk (tiled orders 3-5) */
   int tiledAligned;     /* Tiled: 1 if every tile row stores its own line-aligned window of its output run */
   int itemOrder;        /* Packed/PackedSplit: 0 = a workgroup walks neighbouring slabs, 1 = it keeps its slabs
-                           and walks Mbar positions */
+                           and walks Mbar positions, 2 = the workgroups of an XCD take the items of their
+                           chunk round by round */
   int numPieces;        /* launches per cuttExecute: 1, or the pieces of a tensor of 2^32 elements and more
                            (the other fields then describe the plan of the first piece) */
   int numShapes;        /* different shapes among those pieces (each has a plan of its own): 1..4 */
@@ -164,7 +165,8 @@ long long cuttSlabDecomposition(int rank, const int* dim, const int* permutation
  *   what 2: packed scalars: numThreads, volMbar, itemsPerBlock, padShift, ldsElems, xcdChunk,
  *           elemsPerThread, itemOrder (0: work item w = (m*numSplit1 + s1)*numSplit0 + s0; 1: a
  *           workgroup keeps its slabs, w = ((mb*numSplit1 + s1)*numSplit0 + s0)*itemsPerBlock + mi,
- *           m = mb*itemsPerBlock + mi), then for each of the two split slots: numSplit, slabFloor, slabRem,
+ *           m = mb*itemsPerBlock + mi; 2: numbered as in 0, workgroup q of a chunk of B workgroups takes
+ *           chunkStart + q, chunkStart + q + B, ...), then for each of the two split slots: numSplit, slabFloor, slabRem,
  *           strideIn, strideOut
  *   what 3: class scalars: vol, inCont, outCont
  *   what 4: rowIn[] (vol/inCont input offsets, one per contiguous run)

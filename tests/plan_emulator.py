@@ -113,8 +113,8 @@ def emulate(cands, idx, data):
     off_in, off_out = _mbar_offsets(mbar, vol_mbar)
     ns0, ns1 = splits[0][0], splits[1][0]
     total_items = vol_mbar * ns0 * ns1
-    assert item_order in (0, 1)
-    numbers = total_items if item_order == 0 else -(-vol_mbar // items_per_block) * ns0 * ns1 * items_per_block
+    assert item_order in (0, 1, 2)
+    numbers = total_items if item_order != 1 else -(-vol_mbar // items_per_block) * ns0 * ns1 * items_per_block
     logical_blocks = -(-numbers // items_per_block)
     if xcd_chunk:
         # workgroup b handles logical block (b % 8) * xcd_chunk + b // 8: every logical block once
@@ -124,6 +124,20 @@ def emulate(cands, idx, data):
         assert np.array_equal(np.sort(lb), b)
     else:
         assert info.numBlocks == logical_blocks
+    if item_order == 2:
+        # the numbers are those of order 0, handed out round by round inside each chunk of workgroups:
+        # every number must belong to exactly one workgroup, and to none more than items_per_block
+        chunk_blocks = xcd_chunk if xcd_chunk else info.numBlocks
+        lb = np.arange(info.numBlocks, dtype=np.int64)
+        x, q = lb // chunk_blocks, lb % chunk_blocks
+        start = x * chunk_blocks * items_per_block
+        end = np.minimum(start + chunk_blocks * items_per_block, numbers)
+        taken = []
+        for i in range(items_per_block):
+            w = start + q + i * chunk_blocks
+            taken.append(w[w < end])
+        taken = np.concatenate(taken)
+        assert np.array_equal(np.sort(taken), np.arange(numbers)), "order 2 misses or repeats work items"
     classes = {}
     for c in range(4):
         if ((c & 1) and splits[0][2] == 0) or ((c & 2) and splits[1][2] == 0):
@@ -149,7 +163,7 @@ def emulate(cands, idx, data):
         classes[c] = (in_off[src_p], out_off)
     seen = 0
     for w in range(numbers):
-        if item_order == 0:
+        if item_order != 1:
             t, s0 = divmod(w, ns0)
             m, s1 = divmod(t, ns1)
         else:  # the workgroup keeps its slabs and walks items_per_block Mbar positions

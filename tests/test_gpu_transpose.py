@@ -558,3 +558,36 @@ def test_every_candidate_of_random_midsize_tensors(gpu):
         done += 1
     say("executed %d candidates" % executed)
     assert {"Tiled", "Packed", "PackedSplit"} <= methods
+
+
+def test_work_item_orders_of_the_packed_kernel(gpu):
+    """The three ways of handing work items to workgroups (a workgroup walks neighbouring slabs,
+    keeps its slabs and walks Mbar positions, or takes every B-th item of its XCD's chunk) forced on
+    every Packed / PackedSplit candidate of tensors with even and uneven slabs."""
+    import os
+    import cutt_amd as cutt
+    import oracle
+    cases = [((179, 13, 5, 179, 8), (3, 4, 1, 2, 0)), ((64, 96, 40, 50), (2, 0, 3, 1)), ((31, 549, 2, 3, 9), (3, 0, 2, 4, 1)),
+             ((1000, 7, 300), (2, 1, 0)), ((6, 5, 4, 3, 2, 7, 8, 9), (6, 0, 7, 3, 2, 5, 1, 4))]
+    saved = os.environ.get("CUTT_ITEM_ORDER")
+    seen = {0: 0, 1: 0, 2: 0}
+    try:
+        for dim, perm in cases:
+            for es in (4, 8):
+                data = gpu.seeded(int(np.prod(dim)), es, seed=len(dim))
+                expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
+                for order in (0, 1, 2):
+                    os.environ["CUTT_ITEM_ORDER"] = str(order)
+                    with cutt.Candidates(dim, perm, es) as c:
+                        idx = [i for i in range(len(c)) if c.info(i).method_name in ("Packed", "PackedSplit")]
+                    say("item order %d dim=%s perm=%s es=%d: %d packed candidates" % (order, dim, perm, es, len(idx)))
+                    for i in idx:
+                        info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
+                        assert info.itemOrder == order or (order == 1 and info.itemOrder == 0)  # order 1 needs several Mbar positions
+                        seen[info.itemOrder] += 1
+    finally:
+        if saved is None:
+            os.environ.pop("CUTT_ITEM_ORDER", None)
+        else:
+            os.environ["CUTT_ITEM_ORDER"] = saved
+    assert min(seen.values()) > 20
