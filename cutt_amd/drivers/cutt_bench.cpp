@@ -72,6 +72,8 @@ bool benchTensor(const std::vector<int>& dimIn, const std::vector<int>& permIn) 
   CUTT_CHECK(cuttGetPlanInfo(plan, &info));
   std::printf("method %s blocks %lld threads %d lds %llu candidates %d%s\n", methodNames[info.method], info.numBlocks,
               info.numThreads, info.ldsBytes, info.numCandidates, info.tiledGrouped ? " rows-in-groups" : "");
+  if (info.numPieces > 1)  // a tensor beyond one launch: the line above describes the plan of the first piece
+    std::printf("pieces %d shapes %d\n", info.numPieces, info.numShapes);
   // what the cost model counted for this plan, to set beside hardware counters (128-byte lines)
   std::printf("model: predicted %.1f us, lines read %.0f written %.0f partly written %.0f, LDS cycles %.0f\n", info.usPredicted,
               info.rdLines, info.wrLines, info.wrPartialLines, info.ldsCycles);

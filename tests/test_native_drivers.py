@@ -107,6 +107,19 @@ def test_rank_31_the_highest_rank_that_exists():
 
 
 @pytest.mark.gpu
+def test_more_than_2_to_the_32_elements():
+    # 65552 x 65536 four-byte elements (4.3e9, 17 GB per buffer) transposed: cut into four pieces, one launch
+    # each, checked on the device by closed form (the checker's value pattern repeats every 2^32 elements;
+    # tests/test_gpu_large.py checks the same tensor with a pattern that does not)
+    import os
+    exe = os.path.join(BIN, "cutt_bench")
+    r = subprocess.run([exe, "-elemsize", "4", "-bufelems", "4296015872", "-dim", "65552", "65536", "-permutation", "1", "0",
+                        "-nomemcpy"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=600)
+    assert r.returncode == 0, r.stdout[-2000:]
+    assert "bench OK" in r.stdout and "pieces 4 shapes 1" in r.stdout
+
+
+@pytest.mark.gpu
 def test_tensor_above_4GB_uses_wide_offsets():
     # 671 088 640 doubles = 5.4 GB per buffer: byte offsets no longer fit 32 bits
     import os
