@@ -743,6 +743,7 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
       cur.superAuto = false;
     } else {
       cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
+      cur.itemOrder = plans[best].packed.itemOrder;
     }
     if (plans[best].method == kTiled) {
       cur.tiledGrouped = plans[best].tiled.grouped;
@@ -806,6 +807,17 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
         PlannerOptions v = cur;
         v.maxItemsPerBlock = ipb;
         if (tryVariant(v, true)) cur = v;
+      }
+      // which items a workgroup takes: neighbouring slabs, its own slabs at several Mbar positions,
+      // or every B-th item of its XCD's chunk
+      for (int order : {0, 1, 2}) {
+        if (failed || std::getenv("CUTT_ITEM_ORDER")) break;
+        if (order == start.itemOrder) continue;
+        PlannerOptions v = cur;
+        v.itemOrder = order;
+        Plan probe;
+        if (!rebuildPlan(plans[best], props, v, probe) || probe.packed.itemOrder != order) continue;  // falls back to another order
+        if (tryVariant(v, false)) cur = v;
       }
     }
     // the order in which consecutive work items (or strips of tiles) walk the Mbar ranks decides
