@@ -523,7 +523,8 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
     // back (32 plans: +10 % in the mean, -2 ... +22 %; one item per workgroup +6.5 %, -14 ... +24 %;
     // order 1 +11 % but down to -29 % on other plans, where order 2 is neutral); on other boxes order 0
     // already runs at the estimate and order 2 changes nothing (47 plans: -0.5 ... +1.9 % in the mean).
-    // With 8-byte elements the gain was +2.8 % on the first kind of box: left as it is.
+    // With 8-byte elements the gain was +2.8 % on the first kind of box and -2.5 % on the second (28 changed
+    // plans): left as it is.
     // (Tensors that fit the memory-side cache keep order 0: three of about 5e7 elements ran 5-8 % slower
     // under order 2.)
     const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
