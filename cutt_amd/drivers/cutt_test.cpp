@@ -140,6 +140,48 @@ bool test2(uint64_t seed, int samples) {
   return true;
 }
 
+// Tensors that one launch cannot address are transposed piece by piece (tensors of 2^32 elements and
+// more in production).  CUTT_SPAN_LIMIT lowers the limit, so that random tensors of ordinary size
+// take that path here: both planners, both element sizes, checked like every other tensor.  The
+// reference has no counterpart (its volumes are ints).
+bool test8(uint64_t seed, int samples) {
+  Rng rng(seed + 8);
+  int cut = 0;
+  for (int rank = 2; rank <= 8; rank++) {
+    for (int s = 0; s < std::max(1, samples / 5); s++) {
+      std::vector<int> dim, perm(rank);
+      for (int r = 0; r < rank; r++) perm[r] = r;
+      bool found = false;
+      for (int tries = 0; tries < 100 && !found; tries++) {
+        double vol = 2e5 + 2e7 * rng.uniform();
+        found = randomDims(rng, vol, rank, 0.3, dim);
+      }
+      if (!found) return false;
+      rng.shuffle(perm);
+      const long long vol = volumeOf(dim);
+      const long long limit = vol / 9 + (long long)((double)vol * 0.4 * rng.uniform());
+      setenv("CUTT_SPAN_LIMIT", std::to_string(limit).c_str(), 1);
+      // shapes that cannot be cut (the fastest rank of one side fixed on the other) are refused; skip them
+      cuttHandle probe;
+      cuttResult rc = cuttPlan(&probe, rank, dim.data(), perm.data(), 4, 0);
+      bool ok = true;
+      if (rc == CUTT_SUCCESS) {
+        cuttPlanInfo info;
+        CUTT_CHECK(cuttGetPlanInfo(probe, &info));
+        CUTT_CHECK(cuttDestroy(probe));
+        if (info.numPieces > 1) cut++;
+        ok = testBoth(dim, perm);
+      } else if (rc != CUTT_INVALID_PARAMETER) {
+        ok = false;
+      }
+      unsetenv("CUTT_SPAN_LIMIT");
+      if (!ok) return false;
+    }
+  }
+  std::printf("test8: %d tensors went in pieces\n", cut);
+  return cut > 0;
+}
+
 bool test3() {
   struct Case {
     std::vector<int> dim, perm;
@@ -402,7 +444,7 @@ void usage() {
 int main(int argc, char* argv[]) {
   int gpuid = -1, samples = 100;
   uint64_t seed = 1;
-  std::set<int> tests = {1, 2, 3, 4, 5, 6, 7};
+  std::set<int> tests = {1, 2, 3, 4, 5, 6, 7, 8};
   for (int i = 1; i < argc; i++) {
     std::string a = argv[i];
     if (a == "-device" && i + 1 < argc) {
@@ -439,7 +481,7 @@ int main(int argc, char* argv[]) {
   };
   const Entry entries[] = {{1, "all permutations, ranks 2-7"}, {2, "random tensors, ranks 2-15"}, {3, "hand-picked shapes"},
                            {4, "ten streams"},                 {5, "model counters"},             {6, "refusals and checker"},
-                           {7, "four host threads"}};
+                           {7, "four host threads"},           {8, "tensors cut into pieces"}};
   for (const Entry& e : entries) {
     if (!ok || !tests.count(e.id)) continue;
     std::printf("test %d: %s\n", e.id, e.what);
@@ -452,6 +494,7 @@ int main(int argc, char* argv[]) {
       case 5: ok = test5(seed); break;
       case 6: ok = test6(); break;
       case 7: ok = test7(seed); break;
+      case 8: ok = test8(seed, samples); break;
     }
     std::printf("test %d %s\n", e.id, ok ? "passed" : "FAILED");
     std::fflush(stdout);

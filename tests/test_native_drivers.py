@@ -33,17 +33,17 @@ def test_usage_without_gpu():
 
 @pytest.mark.gpu
 def test_cutt_test_short_run():
-    # all six groups; group 2 with 5 random tensors per rank instead of 100
+    # all eight groups; groups 2 and 8 with fewer random tensors per rank than the full run's 100 and 20
     r = run("cutt_test", "-samples", "5", "-seed", "3", timeout=600)
     assert r.returncode == 0, r.stdout[-2000:]
     assert "test OK" in r.stdout
-    for k in range(1, 7):
+    for k in range(1, 9):
         assert "test %d passed" % k in r.stdout
 
 
 @pytest.mark.gpu
 def test_cutt_test_with_measuring_planner():
-    r = run("cutt_test", "-tests", "3,4,6", "-measure", timeout=600)
+    r = run("cutt_test", "-tests", "3,4,6,8", "-samples", "10", "-measure", timeout=600)
     assert r.returncode == 0, r.stdout[-2000:]
     assert "test OK" in r.stdout
 
