@@ -34,7 +34,7 @@ HBM_PEAK_GBS = 8000.0
 # this run has the signature (method, workgroups, tile order, super-tile shape, cache policy, rows
 # in groups) the profile was taken on, together with the name of the profile; otherwise null.
 C2_TRAFFIC_PROFILES = {
-    ("Tiled", 49152, 5, 4, 8, 3, 0): (3221526426, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
+    ("Tiled", 49152, 5, 2, 8, 3, 0): (3221443482, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
 }
 
 

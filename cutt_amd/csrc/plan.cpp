@@ -570,6 +570,7 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   if (opt.tiledOrder < 0 && tilesM == 2 && tilesK >= 3 && tilesK <= 64 && volMmLastTile <= 24) o.order = 2;
   // Super-tiles of up to superM x superK tiles, shrunk where a direction has fewer tiles.
   int64_t superM = opt.superM, superK = opt.superK;
+  bool gridRule = false;
   if (opt.superAuto && o.order == 5) {
     // Strips that run through all of Mk keep the tiles that share a partly covered line close
     // together.  When all rows start and end on the 128-byte grid on both sides no line is shared
@@ -581,18 +582,27 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
     // to 512 KB apart.  Outside these limits it loses: 4-byte elements -3 % (worst -16 %), rows
     // off the grid -7 %, 10 tiles along Mk cut into 5 + 5 -1...-6 %, fewer than three tiles along
     // Mm -2 %.
+    // Re-measured later, four against two tiles wide where Mm has 16 tiles and more: two wide gained
+    // +0.9 ... +5.7 % on five of six batched transposes of 1024 x 1024-like matrices with an Mbar rank
+    // between the two (C2: 5.53 -> 5.61 TB/s; one -2 %) and +1.3 % in the mean over twelve random tensors
+    // on the grid (-0.8 ... +5.5 %).  Two wide from 8 tiles on, or patches when Mk has exactly 8 tiles,
+    // did not hold up on random tensors (-1 ... -6 % on five of seven; -11 % on (768,64,512,3)/(2,0,1,3)).
     const bool onGrid = rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0;
-    if (onGrid && elemSize == 8 && tilesK >= 16 && tilesM >= 3) {
+    gridRule = onGrid && elemSize == 8 && tilesK >= 16 && tilesM >= 3;
+    if (gridRule) {
       superK = 8;
-      if (tilesM >= 16) superM = 4;
+      if (tilesM >= 16) superM = 2;
     }
   }
-  if (opt.superAuto && (o.order == 5 || o.order == 3) && superM == opt.superM && tilesM > superM && tilesM <= 16) {
+  if (opt.superAuto && !gridRule && (o.order == 5 || o.order == 3) && tilesM > superM && tilesM <= 16 &&
+      !(elemSize == 8 && rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0)) {
     // A rank of 9..16 tiles is not cut into two strips (5 + 4 ... 8 + 8): one strip as wide as the rank
     // reads whole input rows.  Forced Tiled plans on 13 random tensors with such a rank (both widths,
     // with and without Mbar ranks): +2.8 % in the mean, -2 % ... +8 %; the three-rank reversals of the
     // reference's bench 5 with 13 tiles along Mm and 3 along Mk, (817,1480,148)-like: 749 -> 660 us.
-    // From 17 tiles on a single strip gains nothing in the mean (-7 % ... +9 %) and stays cut.
+    // From 17 tiles on a single strip gains nothing in the mean (-7 % ... +9 %) and stays cut.  Not for
+    // 8-byte rows on the line grid: (1024,64,512,6) lost 9 % with one strip of 16, (768,64,1024,4) 4 %, and
+    // twenty random such tensors ran 0.9 % faster cut in two.
     superM = tilesM;
   }
   int64_t sm = std::min<int64_t>(superM, tilesM), sk = std::min<int64_t>(superK, tilesK);
