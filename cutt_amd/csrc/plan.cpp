@@ -556,7 +556,8 @@ struct TileOrdering {
 };
 
 int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
-                    int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, TileOrdering& o) {
+                    int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, bool mbarBetween,
+                    bool beyondCache, TileOrdering& o) {
   // Default: strips of super-tiles, each strip visited for all Mbar positions in turn (order 5;
   // with one Mbar position that is order 3).  The runs of consecutive Mbar positions are usually
   // neighbours in memory, so their shared lines meet in the L2: against finishing one Mbar position
@@ -591,8 +592,26 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
     gridRule = onGrid && elemSize == 8 && tilesK >= 16 && tilesM >= 3;
     if (gridRule) {
       superK = 8;
-      if (tilesM >= 16) superM = 2;
+      // (Two wide only when an Mbar rank lies between Mm and Mk on both sides, as in C2: there the next Mbar
+      // position is the neighbouring row of the same patch.  Batches of separate matrices ran 5 % faster
+      // with patches 8 x 8 than 2 x 8 - twenty random ones, -1 ... +23 % - and tensors with the rank between
+      // were unchanged by the distinction.  Nor for input rows a multiple of 32 KB apart, see below: ten such
+      // tensors with the rank between ran 3.4 % faster 8 wide, -0.6 ... +7 %.)
+      if (tilesM >= 16 && mbarBetween && rowBytesIn % 32768 != 0) superM = 2;
     }
+  }
+  if (opt.superAuto && (o.order == 5 || o.order == 3) && elemSize == 4 && beyondCache && rowBytesIn > 0 &&
+      rowBytesIn % 32768 == 0) {
+    // Input rows a multiple of 32 KB apart (8192 4-byte elements): the 64 rows a tile reads then seem to fall
+    // into the same memory channels (the effect is absent at multiples of 16 KB, so the interleave would
+    // repeat every 32 KB), and a strip of 8 tiles covers only 2 KB of each row.
+    // Strips 16 tiles wide (4 KB per row, what 8-byte elements have anyway) measured +8 ... +15 % on forty
+    // such tensors of 2e8 elements in four layouts (2-D with Mk on and off the line grid, batches, an Mbar
+    // rank between; 12, 24, 32 and 64 wide and patches of 16 x 16 ... 32 x 32 all gained less), on two boxes.
+    // Rows that are multiples of 4, 8 or 16 KB only: -0.3 % (-3 ... +3 %), left alone.  Tensors inside the
+    // memory-side cache lose 1-5 % (8192 x 354 ... 3911); from 0.75 cache sizes per buffer on it pays.
+    gridRule = true;
+    superM = 16;
   }
   if (opt.superAuto && !gridRule && (o.order == 5 || o.order == 3) && tilesM > superM && tilesM <= 16 &&
       !(elemSize == 8 && rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0)) {
@@ -625,7 +644,6 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
 }
 
 bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptions& opt) {
-  (void)props;
   const Split& sp = plan.split;
   const Problem& pb = plan.pb;
   const int64_t tilesM = ceilDiv(sp.volMm, kTile);
@@ -643,8 +661,15 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.tilesK = (int)ceilDiv(sp.volMk + (a.alignedStores ? 128 / pb.elemSize - 1 : 0), kTile);
     a.volMbar = (int)sp.volMbar;
     TileOrdering o;
+    // an Mbar rank that follows Mm in the input and Mk in the output: consecutive Mbar positions are
+    // neighbouring rows on both sides
+    bool between = false;
+    for (int r = 0; r < pb.rank; r++)
+      if (!sp.inMmk[r] && pb.strideIn[r] == sp.volMm && pb.strideOut[r] == sp.volMk) between = true;
+    const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
+    const bool beyondCache = (double)pb.volume * pb.elemSize > 0.75 * cacheBytes;
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
-                                 sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, o);
+                                 sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     a.grouped = opt.tiledGrouped > 0 && !a.alignedStores ? 1 : 0;  // -1: decided from the model's estimate later
@@ -665,7 +690,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     PlannerOptions copt = opt;
     copt.superAuto = false;  // (the measured exceptions are for the Tiled kernel only)
-    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, o);
+    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, o);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;

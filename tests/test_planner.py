@@ -197,6 +197,28 @@ def test_rows_in_groups_only_for_large_unaligned_tensors_of_4_byte_elements(cutt
     assert tiled((31, 97, 101, 659), (3, 1, 2, 0), 4) == 0   # thin tiles: 2 requested lines per line of data
 
 
+def test_super_tile_shapes_of_the_tiled_plan(cutt):
+    def tiled(dim, perm, es):
+        infos, best = method_set(cutt, dim, perm, es)
+        t = [i for i in infos if i.method_name == "Tiled"]
+        assert len(t) == 1
+        return t[0].tiledOrder, t[0].superM, t[0].superK
+    # strips of 8 tiles through all of Mk, every strip for all Mbar positions in turn
+    assert tiled((4457, 44570), (1, 0), 4) == (3, 8, 697)
+    assert tiled((1535, 157, 895), (2, 1, 0), 4) == (5, 8, 14)
+    # 8-byte rows on the 128-byte grid: patches; two wide with an Mbar rank between Mm and Mk (C2)
+    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 8) == (5, 2, 8)
+    assert tiled((2048, 1024, 95), (1, 0, 2), 8) == (5, 8, 8)       # a batch of separate matrices
+    assert tiled((4096, 12, 3936), (2, 1, 0), 8) == (5, 8, 8)       # input rows a multiple of 32 KB
+    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 16, 16)   # 4-byte: one strip for a rank of 16 tiles
+    # 4-byte input rows a multiple of 32 KB apart: strips 16 wide, beyond the memory-side cache only
+    assert tiled((8192, 8192), (1, 0), 4) == (3, 16, 128)
+    assert tiled((16384, 100, 77), (2, 1, 0), 4) == (5, 16, 2)
+    assert tiled((8192, 2048), (1, 0), 4) == (3, 8, 32)
+    assert tiled((4096, 16384), (1, 0), 4) == (3, 8, 256)
+    assert tiled((8192, 8192), (1, 0), 8) == (3, 8, 128)
+
+
 def test_random_shapes_every_candidate(cutt, oracle_mod):
     # Seeded random problems of ranks 2-8 with extents that give several tiles, uneven slabs and
     # fused ranks; every candidate of every problem is replayed on the CPU and compared with the
