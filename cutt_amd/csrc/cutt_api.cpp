@@ -777,8 +777,12 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
       for (const TileKnob& k : {TileKnob{5, 16, 16}, TileKnob{5, 2, 8}, TileKnob{5, 8, 2}, TileKnob{5, 32, 2},
                                 TileKnob{5, 4, 8}, TileKnob{5, 8, 8}, TileKnob{5, 8, 4096}, TileKnob{5, 4, 4096},
                                 TileKnob{1, 8, 4096}, TileKnob{2, 8, 4096}, TileKnob{3, 8, 4096},
-                                TileKnob{3, 16, 16}}) {
+                                TileKnob{3, 16, 16},
+                                // small patches in order 6 (batched transposes of power-of-two sizes: up to +15 %)
+                                TileKnob{6, 2, 2}, TileKnob{6, 1, 1}, TileKnob{6, 2, 1}, TileKnob{6, 1, 2},
+                                TileKnob{6, 2, 4}, TileKnob{6, 4, 2}, TileKnob{6, 4, 4}, TileKnob{6, 1, 4}}) {
         if (failed) break;
+        if (k.order == 6 && plans[best].split.volMbar <= 1) continue;
         if (k.order == start.tiledOrder && k.superM == start.superM && k.superK == start.superK) continue;
         PlannerOptions v = cur;
         v.tiledOrder = k.order; v.superM = k.superM; v.superK = k.superK;

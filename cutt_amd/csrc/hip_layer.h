@@ -107,7 +107,9 @@ typedef struct cuttHipTiledArgs {
   int order;          /* logical numbering of the workgroups: 0 = Mbar fastest, 1 = tiles along Mm
                          fastest, 2 = tiles along Mk fastest, 3 / 4 = superM x superK super-tiles with the
                          tiles along Mm / along Mk running fastest inside and between them; 5 = as 3,
-                         but every super-tile is visited for all Mbar positions in turn */
+                         but every super-tile is visited for all Mbar positions in turn; 6 = as 5 with
+                         the super-tiles numbered along Mk first and each row of them rotated by its
+                         index along Mm (the XCDs then work on different columns at one time) */
   uint32_t xcdChunk;  /* 0: workgroup b is logical position b; else (b % 8)*xcdChunk + b/8, and the
                          grid has 8*xcdChunk workgroups */
   uint32_t superM, superK;

@@ -615,7 +615,7 @@ extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || (a->alignedStores != 0 && a->alignedStores != 1) ||
       a->tilesK != (a->volMk + (a->alignedStores ? 128 / a->elemSize - 1 : 0) + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 5 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1) ||
+      a->order < 0 || a->order > 6 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1) ||
       (a->alignedStores && a->grouped))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
@@ -656,7 +656,7 @@ extern "C" int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 5 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 6 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
   if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))

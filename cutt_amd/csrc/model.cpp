@@ -350,7 +350,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const int order = copy ? plan.tcopy.order : plan.tiled.order;
     auto mbarDist = [&](int rank, bool input) -> double {
       // order 5 walks the Mbar positions strip by strip, the others tensor slice by tensor slice
-      double d = order == 5 ? std::min(superM, tilesM) * tilesK : tilesM * tilesK;
+      double d = order >= 5 ? std::min(superM, tilesM) * tilesK : tilesM * tilesK;
       for (int k = 0; k < mb.n; k++) {
         const bool hit = input ? mb.d[k].strideIn == (uint32_t)pb.strideIn[rank]
                                : mb.d[k].strideOut == (uint32_t)pb.strideOut[rank];

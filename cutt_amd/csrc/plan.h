@@ -145,7 +145,7 @@ struct Plan {
 struct PlannerOptions {
   int forceMethod = 0;      // 0 = all methods, else only this Method (Trivial always allowed)
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
-  int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3-5: strips of 8 tiles along Mm
+  int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3-6: strips of 8 tiles along Mm
   bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
   int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time

@@ -55,7 +55,7 @@ typedef struct cuttPlanInfo {
    * runs, on the read and on the write side (0 = no such neighbour) */
   double rdEdgeDist, wrEdgeDist;
   int tiledGrouped;     /* Tiled: 1 if a lane keeps 4 instead of 16 tile rows in flight */
-  int superM, superK;   /* Tiled/TiledCopy: shape of the super-tiles the workgroups walk (tiled orders 3-5) */
+  int superM, superK;   /* Tiled/TiledCopy: shape of the super-tiles the workgroups walk (tiled orders 3-6) */
   int tiledAligned;     /* Tiled: 1 if every tile row stores its own line-aligned window of its output run */
   int itemOrder;        /* Packed/PackedSplit: 0 = a workgroup walks neighbouring slabs, 1 = it keeps its slabs
                            and walks Mbar positions, 2 = the workgroups of an XCD take the items of their

@@ -46,15 +46,19 @@ def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk,
         m, tm = t // tiles_m, t % tiles_m
         ok = m < vol_mbar
     else:
-        assert order in (3, 4, 5) and sup_m >= 1 and sup_k >= 1
+        assert order in (3, 4, 5, 6) and sup_m >= 1 and sup_k >= 1
         n_sm, n_sk = -(-tiles_m // sup_m), -(-tiles_k // sup_k)
         per = sup_m * sup_k
         w, t = l % per, l // per
-        if order == 5:
+        if order >= 5:
             st, m = t // vol_mbar, t % vol_mbar
         else:
             st, m = t % (n_sm * n_sk), t // (n_sm * n_sk)
-        if order != 4:
+        if order == 6:
+            mi = st // n_sk
+            tm = mi * sup_m + w % sup_m
+            tk = ((st % n_sk + mi) % n_sk) * sup_k + w // sup_m
+        elif order != 4:
             tm = (st % n_sm) * sup_m + w % sup_m
             tk = (st // n_sm) * sup_k + w // sup_m
         else:

@@ -591,3 +591,32 @@ def test_work_item_orders_of_the_packed_kernel(gpu):
         else:
             os.environ["CUTT_ITEM_ORDER"] = saved
     assert min(seen.values()) > 20
+
+
+def test_tile_orders_and_patch_shapes_of_the_tiled_kernels(gpu, monkeypatch):
+    """Every numbering of the tiled kernels' workgroups (orders 0-6) with several super-tile shapes, on shapes
+    with edge tiles, several Mbar ranks and a leading rank that stays (TiledCopy), both widths."""
+    import cutt_amd as cutt
+    import oracle
+    cases = [((130, 9, 70), (2, 1, 0)), ((200, 3, 5, 333), (3, 1, 2, 0)), ((1000, 30, 777), (2, 1, 0)), ((64, 64), (1, 0)),
+             ((257, 129, 6), (1, 0, 2)), ((150, 7, 300), (0, 2, 1)), ((512, 12, 512, 3), (2, 1, 0, 3))]
+    shapes = [(1, 1), (2, 2), (3, 5), (8, 4096), (4, 1), (1, 4)]
+    seen = set()
+    for dim, perm in cases:
+        for es in (4, 8):
+            data = gpu.seeded(int(np.prod(dim)), es, seed=len(dim) + es)
+            expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
+            for order in range(7):
+                for sm, sk in (shapes if order >= 3 else shapes[:1]):
+                    monkeypatch.setenv("CUTT_TILED_ORDER", str(order))
+                    monkeypatch.setenv("CUTT_SUPER_M", str(sm))
+                    monkeypatch.setenv("CUTT_SUPER_K", str(sk))
+                    with cutt.Candidates(dim, perm, es) as c:
+                        idx = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]
+                    assert idx, (dim, perm)
+                    for i in idx:
+                        info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
+                        assert info.tiledOrder == order
+                        seen.add((info.method_name, order))
+        say("tile orders dim=%s perm=%s done" % (dim, perm))
+    assert {("Tiled", o) for o in range(7)} <= seen and {("TiledCopy", o) for o in range(7)} <= seen

@@ -219,6 +219,27 @@ def test_super_tile_shapes_of_the_tiled_plan(cutt):
     assert tiled((8192, 8192), (1, 0), 8) == (3, 8, 128)
 
 
+def test_every_tile_order_visits_every_tile_once(cutt, oracle_mod, monkeypatch):
+    # orders 0-6 of the tiled kernels with several super-tile shapes, replayed on the CPU
+    import plan_emulator as pe
+    for dim, perm in [((130, 9, 70), (2, 1, 0)), ((200, 3, 5, 33), (3, 1, 2, 0)), ((150, 7, 300), (0, 2, 1)), ((257, 129, 6), (1, 0, 2))]:
+        for es in (4, 8):
+            data = np.arange(int(np.prod(dim)), dtype=np.uint32 if es == 4 else np.uint64)
+            expect = oracle_mod.transpose(list(dim), list(perm), data)
+            for order in range(7):
+                for sm, sk in ((1, 1), (2, 2), (3, 5), (8, 4096)):
+                    monkeypatch.setenv("CUTT_TILED_ORDER", str(order))
+                    monkeypatch.setenv("CUTT_SUPER_M", str(sm))
+                    monkeypatch.setenv("CUTT_SUPER_K", str(sk))
+                    with cutt.Candidates(list(dim), list(perm), es) as c:
+                        tiled = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]
+                        assert tiled
+                        for i in tiled:
+                            assert c.info(i).tiledOrder == order
+                            out, count = pe.emulate(c, i, data)
+                            assert np.array_equal(out, expect) and (count == 1).all(), (dim, perm, es, order, sm, sk)
+
+
 def test_random_shapes_every_candidate(cutt, oracle_mod):
     # Seeded random problems of ranks 2-8 with extents that give several tiles, uneven slabs and
     # fused ranks; every candidate of every problem is replayed on the CPU and compared with the
