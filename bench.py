@@ -35,6 +35,7 @@ HBM_PEAK_GBS = 8000.0
 # in groups) the profile was taken on, together with the name of the profile; otherwise null.
 C2_TRAFFIC_PROFILES = {
     ("Tiled", 49152, 5, 2, 8, 3, 0): (3221443482, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
+    ("Tiled", 49152, 6, 2, 2, 3, 0): (3221508198, "profiles/tiledKernel_u64_C2_order6_measured_plan.txt"),
 }
 
 
