@@ -833,6 +833,13 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
       v.mbarOrder = order;
       if (tryVariant(v, false)) cur = v;
     }
+    // workgroup b at logical position b (the XCDs then interleave instead of walking a chunk each):
+    // rarely better, but then by 5-10 % (measured on PackedSplit plans with long runs)
+    if (!failed && !std::getenv("CUTT_XCD_AWARE") && cur.xcdAware) {
+      PlannerOptions v = cur;
+      v.xcdAware = false;
+      if (tryVariant(v, false)) cur = v;
+    }
     // ... and the other cache policies of the global accesses
     for (int pol : {0, 1, 3}) {
       if (failed || std::getenv("CUTT_CACHE_POLICY")) break;
