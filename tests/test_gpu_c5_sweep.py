@@ -48,9 +48,10 @@ def test_sweep_both_planners_every_tensor():
     worst_heuristic = min(fp64, key=lambda r: r["plan"]["pct"])
     assert worst_measured["measure"]["pct"] >= 70.0, worst_measured
     assert worst_heuristic["plan"]["pct"] >= 70.0, worst_heuristic
-    # the measuring planner must not end up behind the heuristic one by more than timing noise
+    # the measuring planner must not end up behind the heuristic one by more than timing noise (the same plan
+    # timed twice in one process differs by up to 9 % here: the first launch after an idle gap runs faster)
     for r in results:
-        assert r["measure"]["ms"] <= 1.08 * r["plan"]["ms"], r
+        assert r["measure"]["ms"] <= 1.12 * r["plan"]["ms"], r
 
 
 @pytest.mark.parametrize("index", [0, 9, 18, 27, 36, 45])
