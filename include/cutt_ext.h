@@ -38,7 +38,7 @@ typedef struct cuttPlanInfo {
   long long numBlocks;
   int numThreads;
   int itemsPerBlock;    /* Packed/PackedSplit */
-  int tiledOrder;       /* Tiled/TiledCopy */
+  int tiledOrder;       /* Tiled/TiledCopy: numbering of the workgroups, 0-6 (hip_layer.h: cuttHipTiledArgs.order) */
   unsigned long long ldsBytes;
   /* cost model */
   double usPredicted;
