@@ -569,8 +569,9 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   // fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows are written as
   // streams - as long as the two tiles that share an input row stay close (at most 64 tiles along Mk).
   // With 4-byte elements that holds up to a 104-wide rank (ten three-rank tensors with a leading rank of
-  // 89..104, batches and reversals: +1 ... +21 %, all ten faster; 110..126 wide: -7 ... +4 %; 8-byte
-  // elements beyond 88: +2 % in the mean, left alone).
+  // 89..104, batches and reversals: +1 ... +21 %, all ten faster; a second set of 24 on another box: +3 % in
+  // the mean, -9 ... +8 %, 19 faster; 110..126 wide: -7 ... +4 %; 8-byte elements beyond 88: +2 % in the
+  // mean, left alone).
   if (opt.tiledOrder < 0 && tilesM == 2 && tilesK >= 3 && tilesK <= 64 && volMmLastTile <= (elemSize == 4 ? 40 : 24))
     o.order = 2;
   // Super-tiles of up to superM x superK tiles, shrunk where a direction has fewer tiles.
