@@ -102,49 +102,65 @@ __device__ __forceinline__ void countAccess(LaneCounts& c, bool write, bool idle
   c.v[write ? kWrSectors : kRdSectors] += waveDistinct(byte >> 5);
 }
 
-template <bool COPY, typename Args>
-__global__ __launch_bounds__(kTileThreads) void countTiledKernel(const Args a, uint32_t strideOut, unsigned long long* total) {
+// Mirrors tiledKernel: the tile order, the Mbar decode and the lanes' row addresses come from the
+// functions that kernel uses (tile_order.h: decodeTile, tileLanes, tileReadElem, tileWriteElem).
+template <bool FUSED>
+__global__ __launch_bounds__(kTileThreads) void countTiledKernel(const cuttHipTiledArgs a, unsigned long long* total) {
   uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
   const uint32_t es = (uint32_t)a.elemSize, words = es / 4;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const TileLanes t = tileLanes<FUSED>(a, tm, tk, offIn, offOut, lane, wave);
+  LaneCounts c = {};
+  // reads: lanes along the input-contiguous axis, rows along Mk
+  for (int j = 0; j < kTileRows; j++) {
+    if ((uint32_t)(j / kGroupRows) >= t.groupsK) continue;
+    const uint32_t row = wave + kWaves * j, r = min(row, t.wK);
+    countAccess(c, false, row > t.wK, tileReadElem<FUSED>(t, a, wave, j), es);
+    if (row <= t.wK) c.maxDegree = max(c.maxDegree, waveMaxMultiplicity(((r * (kTile + 1) + t.cx) * words) & 63, __ballot(lane <= t.wM)));
+  }
+  // writes: lanes along the output-contiguous axis, rows along Mm
+  for (int j = 0; j < kTileRows; j++) {
+    if ((uint32_t)(j / kGroupRows) >= t.groupsM) continue;
+    const uint32_t row = wave + kWaves * j, r = min(row, t.wM);
+    const uint32_t elem = tileWriteElem<FUSED>(t, a, wave, j);
+    countAccess(c, true, row > t.wM, elem, es);
+    if (row <= t.wM) c.maxDegree = max(c.maxDegree, waveMaxMultiplicity(((t.ck * (kTile + 1) + r) * words) & 63, __ballot(lane <= t.wK)));
+    // lane 0 holds the first element of the row's run inside this tile
+    if (row <= t.wM && lane == 0) c.v[kWrPartial] += partialEnds(elem, t.wK + 1, es);
+  }
+  // the partial-line counts sit in lane 0 already; the per-instruction counts are wave-uniform
+  flush(c, total);
+}
+
+// Mirrors tiledCopyKernel (its whole address arithmetic is the three lines below).
+__global__ __launch_bounds__(kTileThreads) void countTiledCopyKernel(const cuttHipTiledCopyArgs a, unsigned long long* total) {
+  uint32_t tm, tk, m;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  uint32_t offIn, offOut;
+  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  const uint32_t es = (uint32_t)a.elemSize;
+  const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t m0 = tm * kTile, k0 = tk * kTile;
   const uint32_t wM = min((uint32_t)kTile, (uint32_t)a.volMm - m0) - 1;
   const uint32_t wK = min((uint32_t)kTile, (uint32_t)a.volMk - k0) - 1;
-  const uint32_t groupsK = (wK >> 4) + 1, groupsM = (wM >> 4) + 1;
-  LaneCounts c = {};
-  // reads: lanes along input rank 0, rows along the Mk rank
+  const uint32_t groupsK = (wK >> 4) + 1;
   const uint32_t cx = min(lane, wM);
+  LaneCounts c = {};
   for (int j = 0; j < kTileRows; j++) {
     if ((uint32_t)(j / kGroupRows) >= groupsK) continue;
     const uint32_t row = wave + kWaves * j, r = min(row, wK);
     countAccess(c, false, row > wK, (uint64_t)offIn + m0 + cx + (uint64_t)(k0 + r) * a.strideInK, es);
-    if (!COPY && row <= wK) c.maxDegree = max(c.maxDegree, waveMaxMultiplicity(((r * (kTile + 1) + cx) * words) & 63, __ballot(lane <= wM)));
   }
-  if (COPY) {
-    // writes: the same rows, lanes along rank 0 again
-    for (int j = 0; j < kTileRows; j++) {
-      if ((uint32_t)(j / kGroupRows) >= groupsK) continue;
-      const uint32_t row = wave + kWaves * j, r = min(row, wK);
-      const uint64_t start = (uint64_t)offOut + m0 + (uint64_t)(k0 + r) * strideOut;
-      countAccess(c, true, row > wK, start + cx, es);
-      if (row <= wK && lane == 0) c.v[kWrPartial] += partialEnds(start, wM + 1, es);
-    }
-  } else {
-    // writes: lanes along the Mk rank, rows along rank 0
-    const uint32_t ck = min(lane, wK);
-    for (int j = 0; j < kTileRows; j++) {
-      if ((uint32_t)(j / kGroupRows) >= groupsM) continue;
-      const uint32_t row = wave + kWaves * j, r = min(row, wM);
-      const uint64_t start = (uint64_t)offOut + k0 + (uint64_t)(m0 + r) * strideOut;
-      countAccess(c, true, row > wM, start + ck, es);
-      if (row <= wM) c.maxDegree = max(c.maxDegree, waveMaxMultiplicity(((ck * (kTile + 1) + r) * words) & 63, __ballot(lane <= wK)));
-      if (row <= wM && lane == 0) c.v[kWrPartial] += partialEnds(start, wK + 1, es);
-    }
+  for (int j = 0; j < kTileRows; j++) {
+    if ((uint32_t)(j / kGroupRows) >= groupsK) continue;
+    const uint32_t row = wave + kWaves * j, r = min(row, wK);
+    const uint64_t start = (uint64_t)offOut + m0 + (uint64_t)(k0 + r) * a.strideOutK;
+    countAccess(c, true, row > wK, start + cx, es);
+    if (row <= wK && lane == 0) c.v[kWrPartial] += partialEnds(start, wM + 1, es);
   }
-  // the partial-line counts sit in lane 0 already; the per-instruction counts are wave-uniform
   flush(c, total);
 }
 
@@ -245,23 +261,21 @@ int runCount(cuttHipStreamCounts* out, void* stream, F&& launch) {
 extern "C" int cuttHipCountTiled(const cuttHipTiledArgs* a, cuttHipStreamCounts* out, void* stream) {
   if (int v = cuttHipValidateTiled(a); v != 0) return v;
   if (a->alignedStores) return (int)hipErrorNotSupported;
-  const uint64_t blocks = a->xcdChunk ? (uint64_t)a->xcdChunk * kNumXcd
-                                      : (a->order >= 3 ? (uint64_t)((a->tilesM + a->superM - 1) / a->superM) *
-                                                             ((a->tilesK + a->superK - 1) / a->superK) * a->superM * a->superK * (uint64_t)a->volMbar
-                                                       : (uint64_t)a->tilesM * a->tilesK * (uint64_t)a->volMbar);
+  const long long blocks = cuttHipTiledGrid(a);
+  if (blocks < 1) return (int)hipErrorInvalidConfiguration;
+  const bool fused = a->rowsK.n > 0 || a->rowsM.n > 0;
   return runCount(out, stream, [&](unsigned long long* d, hipStream_t s) {
-    return launchCount(countTiledKernel<false, cuttHipTiledArgs>, dim3((uint32_t)blocks), dim3(kTileThreads), s, *a, a->strideOutM, d);
+    return fused ? launchCount(countTiledKernel<true>, dim3((uint32_t)blocks), dim3(kTileThreads), s, *a, d)
+                 : launchCount(countTiledKernel<false>, dim3((uint32_t)blocks), dim3(kTileThreads), s, *a, d);
   });
 }
 
 extern "C" int cuttHipCountTiledCopy(const cuttHipTiledCopyArgs* a, cuttHipStreamCounts* out, void* stream) {
   if (int v = cuttHipValidateTiledCopy(a); v != 0) return v;
-  const uint64_t blocks = a->xcdChunk ? (uint64_t)a->xcdChunk * kNumXcd
-                                      : (a->order >= 3 ? (uint64_t)((a->tilesM + a->superM - 1) / a->superM) *
-                                                             ((a->tilesK + a->superK - 1) / a->superK) * a->superM * a->superK * (uint64_t)a->volMbar
-                                                       : (uint64_t)a->tilesM * a->tilesK * (uint64_t)a->volMbar);
+  const long long blocks = cuttHipTiledCopyGrid(a);
+  if (blocks < 1) return (int)hipErrorInvalidConfiguration;
   return runCount(out, stream, [&](unsigned long long* d, hipStream_t s) {
-    return launchCount(countTiledKernel<true, cuttHipTiledCopyArgs>, dim3((uint32_t)blocks), dim3(kTileThreads), s, *a, a->strideOutK, d);
+    return launchCount(countTiledCopyKernel, dim3((uint32_t)blocks), dim3(kTileThreads), s, *a, d);
   });
 }
 

@@ -86,7 +86,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_TILED_FUSE"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
@@ -415,6 +415,8 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_SUPER_K")) { opt.superK = std::max(1, std::atoi(e)); opt.superAuto = false; }
   if (const char* e = std::getenv("CUTT_TILED_GROUPED")) opt.tiledGrouped = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILED_ALIGNED")) opt.tiledAligned = std::atoi(e) != 0 ? 1 : 0;
+  if (const char* e = std::getenv("CUTT_TILE_DIGITS")) opt.tileDigits = e;
+  if (const char* e = std::getenv("CUTT_TILED_FUSE")) opt.tiledFuse = std::atoi(e) != 0 ? 1 : 0;
   return opt;
 }
 
@@ -1202,6 +1204,26 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
     case 6:
       if (!packed) return -1;
       v.assign(p.tab[cls].shIdx.begin(), p.tab[cls].shIdx.end());
+      break;
+    case 7:  // Tiled: (extent, stride) of the ranks a tile axis runs over: cls 0 = Mk (input strides), 1 = Mm (output strides)
+      if (p.method != kTiled || cls > 1) return -1;
+      {
+        const cuttHipRowRadix& rr = cls == 0 ? p.tiled.rowsK : p.tiled.rowsM;
+        for (int k = 0; k < rr.n; k++) {
+          v.push_back(rr.extent[k]);
+          v.push_back(rr.stride[k]);
+        }
+      }
+      break;
+    case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix) of the digits, fastest first
+      if (p.method != kTiled && p.method != kTiledCopy) return -1;
+      {
+        const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
+        for (int k = 0; k < dg.n; k++) {
+          v.push_back(dg.d[k].which);
+          v.push_back(dg.d[k].radix);
+        }
+      }
       break;
     default:
       return -1;

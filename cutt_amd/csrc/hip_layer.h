@@ -92,10 +92,47 @@ uint32_t cuttHipDivide(uint32_t n, cuttHipDivisor dv);
 int cuttHipFinishMbar(cuttHipMbar* mb);
 
 /*
- * Tiled method: a batch of 2-D transposes between input rank 0 (extent volMm,
- * input stride 1, output stride strideOutM) and the rank that leads the
- * output (extent volMk, input stride strideInK, output stride 1), staged
- * through a padded 64x64 LDS tile.  One workgroup per (tile, Mbar position).
+ * A free numbering of the workgroups of a tiled launch (tile order 7): the logical workgroup index is
+ * read as a mixed-radix number, first digit fastest, and every digit belongs to one of the three
+ * coordinates of a workgroup - tile along Mm (which = 0), tile along Mk (1), Mbar position (2).  A
+ * coordinate is the mixed-radix number of its own digits in the order they appear.  The product of a
+ * coordinate's radices must reach its extent; indices whose coordinates fall beyond an extent are
+ * padding workgroups.  Orders 0-5 are special cases (patches of 2 x 8 tiles walked for 192 Mbar
+ * positions in turn: m2 k8 b192 m8 k2 for 16 x 16 tiles).
+ */
+#define CUTT_MAX_TILE_DIGITS 12
+typedef struct cuttHipTileDigit {
+  uint32_t radix;
+  uint32_t which;       /* 0 tile along Mm, 1 tile along Mk, 2 Mbar position */
+  cuttHipDivisor div;   /* division by radix (cuttHipMakeDivisor) */
+} cuttHipTileDigit;
+
+typedef struct cuttHipTileDigits {
+  int n;
+  cuttHipTileDigit d[CUTT_MAX_TILE_DIGITS];
+} cuttHipTileDigits;
+
+/*
+ * Offsets of the rows of a tile when a tile axis runs over several fused ranks: row index i along the
+ * set (first rank fastest) has the offset sum_k ((i / prod_{j<k} extent_j) % extent_k) * stride_k.
+ * n = 0: the axis is a single rank and the offset is i * stride (strideInK / strideOutM of the
+ * arguments).
+ */
+#define CUTT_MAX_TILE_SET 4
+typedef struct cuttHipRowRadix {
+  int n;
+  uint32_t extent[CUTT_MAX_TILE_SET];
+  uint32_t stride[CUTT_MAX_TILE_SET];
+  cuttHipDivisor div[CUTT_MAX_TILE_SET]; /* division by extent[k] */
+} cuttHipRowRadix;
+
+/*
+ * Tiled method: a batch of 2-D transposes between the ranks that lead the input (Mm: fused extent
+ * volMm, contiguous in the input) and the ranks that lead the output (Mk: fused extent volMk,
+ * contiguous in the output), staged through a padded 64x64 LDS tile.  One workgroup per (tile, Mbar
+ * position).  With one rank on each side (rowsK.n == rowsM.n == 0) row k of a tile lies
+ * k * strideInK into the input and row m lies m * strideOutM into the output; with several ranks on a
+ * side the rows' offsets follow rowsK / rowsM.
  */
 typedef struct cuttHipTiledArgs {
   int elemSize;       /* 4 or 8 */
@@ -109,7 +146,8 @@ typedef struct cuttHipTiledArgs {
                          tiles along Mm / along Mk running fastest inside and between them; 5 = as 3,
                          but every super-tile is visited for all Mbar positions in turn; 6 = as 5 with
                          the super-tiles numbered along Mk first and each row of them rotated by its
-                         index along Mm (the XCDs then work on different columns at one time) */
+                         index along Mm (the XCDs then work on different columns at one time); 7 = the
+                         mixed-radix numbering in `digits` */
   uint32_t xcdChunk;  /* 0: workgroup b is logical position b; else (b % 8)*xcdChunk + b/8, and the
                          grid has 8*xcdChunk workgroups */
   uint32_t superM, superK;
@@ -119,6 +157,9 @@ typedef struct cuttHipTiledArgs {
   int alignedStores;  /* 1: every tile row stores its own 64-element window of the output run, shifted
                          so that it starts on a 128-byte line; tilesK is then
                          ceil((volMk + 128/elemSize - 1) / 64) and grouped must be 0 */
+  cuttHipRowRadix rowsK; /* Mk index -> input offset (n == 0: index * strideInK) */
+  cuttHipRowRadix rowsM; /* Mm index -> output offset (n == 0: index * strideOutM) */
+  cuttHipTileDigits digits; /* order 7 only */
   cuttHipMbar mbar;
 } cuttHipTiledArgs;
 
@@ -138,6 +179,7 @@ typedef struct cuttHipTiledCopyArgs {
   uint32_t xcdChunk;
   uint32_t superM, superK;
   int cachePolicy;
+  cuttHipTileDigits digits; /* order 7 only */
   cuttHipMbar mbar;
 } cuttHipTiledCopyArgs;
 
@@ -250,6 +292,9 @@ const char* cuttHipErrorString(int err);
 int cuttHipValidateTiled(const cuttHipTiledArgs* args);
 int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* args);
 int cuttHipValidatePacked(const cuttHipPackedArgs* args);
+/* Workgroups of a tiled launch with these arguments (padding workgroups included), 0 if they have no valid grid. */
+long long cuttHipTiledGrid(const cuttHipTiledArgs* args);
+long long cuttHipTiledCopyGrid(const cuttHipTiledCopyArgs* args);
 int cuttHipLaunchTiled(const cuttHipTiledArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* args, const void* in, void* out, void* stream);
 int cuttHipLaunchPacked(const cuttHipPackedArgs* args, const void* in, void* out, void* stream);

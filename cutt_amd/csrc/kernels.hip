@@ -74,53 +74,41 @@ __device__ __forceinline__ void waitForGlobalAccesses() { asm volatile("s_waitcn
 // elements, large tensors) it is 3-11 % faster: the neighbouring tiles' requests for a shared line
 // then arrive while the line is still in the L2.  On aligned or cache-resident tensors it is up to
 // 10 % slower, so the planner decides (cuttHipTiledArgs.grouped).
-template <typename T, int NT, bool GROUPED>
+//
+// FUSED: a tile axis runs over several fused ranks (the ranks that lead the input on the Mm side, the
+// ranks that lead the output on the Mk side), so the rows of a tile are not equally far apart.  Lane l
+// derives the offset of row l of either axis with a short mixed-radix decode (tileRowOffsets) and the
+// wave picks a row's offset out of that lane; the elements of a row are contiguous as before.
+template <typename T, int NT, bool GROUPED, bool FUSED>
 __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledArgs a,
                                                             const T* __restrict__ in,
                                                             T* __restrict__ out) {
   __shared__ T tile[kTile][kTile + 1];
 
   uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
-  const uint32_t m0 = tm * kTile, k0 = tk * kTile;
-  const uint32_t volMm = a.volMm, volMk = a.volMk;
+  // tile geometry, clamped edges, skipped row groups: tile_order.h
+  const TileLanes t = tileLanes<FUSED>(a, tm, tk, offIn, offOut, lane, wave);
 
-  // Edge tiles are handled without branches: indices are clamped to the last valid row / column,
-  // so out-of-range lanes repeat the access of the edge element (same address, same value).  That
-  // keeps the loop bodies straight-line code, and all 16 loads of a lane go out back to back.
-  const uint32_t wM = min((uint32_t)kTile, volMm - m0) - 1;  // last valid column / row inside the tile
-  const uint32_t wK = min((uint32_t)kTile, volMk - k0) - 1;
-
-  // The 16 rows of a lane come in kRowGroups groups of 4; group g covers tile rows 16g..16g+15
-  // over the four waves.  An edge tile skips the groups that lie entirely beyond its valid part
-  // (a test that is uniform over the workgroup), so that a thin edge costs a quarter of a tile's
-  // instructions, not all of them; inside a group the clamping above still applies.
-  const uint32_t groupsK = (wK >> 4) + 1, groupsM = (wM >> 4) + 1;
-
-  // Read: lanes run along input rank 0, rows along the Mk rank.
+  // Read: lanes run along the input-contiguous axis (Mm), rows along Mk.
   {
-    const uint32_t cx = min(lane, wM);
-    const T* src = in + (offIn + m0 + cx);
     T v[kTileRows];
 #pragma unroll
     for (int g = 0; g < kRowGroups; g++) {
-      if ((uint32_t)g < groupsK) {
+      if ((uint32_t)g < t.groupsK) {
 #pragma unroll
-        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-          const uint32_t r = min(wave + kWaves * j, wK);
-          v[j] = ldg<NT>(src + (k0 + r) * a.strideInK);
-        }
+        for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) v[j] = ldg<NT>(in + tileReadElem<FUSED>(t, a, wave, j));
         if constexpr (GROUPED) {
           waitForGlobalAccesses();
 #pragma unroll
           for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-            const uint32_t r = min(wave + kWaves * j, wK);
-            tile[r][cx] = v[j];
+            const uint32_t r = min(wave + kWaves * j, t.wK);
+            tile[r][t.cx] = v[j];
           }
         }
       }
@@ -128,36 +116,31 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
     if constexpr (!GROUPED) {
 #pragma unroll
       for (int g = 0; g < kRowGroups; g++) {
-        if ((uint32_t)g < groupsK) {
+        if ((uint32_t)g < t.groupsK) {
 #pragma unroll
           for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-            const uint32_t r = min(wave + kWaves * j, wK);
-            tile[r][cx] = v[j];
+            const uint32_t r = min(wave + kWaves * j, t.wK);
+            tile[r][t.cx] = v[j];
           }
         }
       }
     }
   }
   __syncthreads();
-  // Write: lanes run along the Mk rank (contiguous in the output).
+  // Write: lanes run along the output-contiguous axis (Mk), rows along Mm.
   {
-    const uint32_t ck = min(lane, wK);
-    T* dst = out + (offOut + k0 + ck);
     T v[kTileRows];
 #pragma unroll
     for (int g = 0; g < kRowGroups; g++) {
-      if ((uint32_t)g < groupsM) {
+      if ((uint32_t)g < t.groupsM) {
 #pragma unroll
         for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-          const uint32_t r = min(wave + kWaves * j, wM);
-          v[j] = tile[ck][r];
+          const uint32_t r = min(wave + kWaves * j, t.wM);
+          v[j] = tile[t.ck][r];
         }
         if constexpr (GROUPED) {
 #pragma unroll
-          for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-            const uint32_t r = min(wave + kWaves * j, wM);
-            stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
-          }
+          for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) stg<NT>(out + tileWriteElem<FUSED>(t, a, wave, j), v[j]);
           waitForGlobalAccesses();
         }
       }
@@ -165,12 +148,9 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
     if constexpr (!GROUPED) {
 #pragma unroll
       for (int g = 0; g < kRowGroups; g++) {
-        if ((uint32_t)g < groupsM) {
+        if ((uint32_t)g < t.groupsM) {
 #pragma unroll
-          for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) {
-            const uint32_t r = min(wave + kWaves * j, wM);
-            stg<NT>(dst + (m0 + r) * a.strideOutM, v[j]);
-          }
+          for (int j = g * kGroupRows; j < (g + 1) * kGroupRows; j++) stg<NT>(out + tileWriteElem<FUSED>(t, a, wave, j), v[j]);
         }
       }
     }
@@ -202,7 +182,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledAlignedKernel(const cuttHip
   __shared__ T tile[ROWS][kTile + 1];
 
   uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
 
@@ -281,7 +261,7 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
                                                                 const T* __restrict__ in,
                                                                 T* __restrict__ out) {
   uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
   uint32_t offIn, offOut;
   mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
 
@@ -517,9 +497,21 @@ bool divisorOk(const cuttHipDivisor& dv, uint32_t d) {
 
 // Number of workgroups of a tiled launch; checks the ordering parameters.
 bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk, uint32_t superM,
-              uint32_t superK, uint64_t& blocks) {
+              uint32_t superK, const cuttHipTileDigits& dg, uint64_t& blocks) {
   uint64_t logical = (uint64_t)tilesM * tilesK * (uint64_t)volMbar;
-  if (order >= 3) {
+  if (order == 7) {
+    if (dg.n < 1 || dg.n > CUTT_MAX_TILE_DIGITS) return false;
+    uint64_t span[3] = {1, 1, 1};
+    logical = 1;
+    for (int i = 0; i < dg.n; i++) {
+      const cuttHipTileDigit& d = dg.d[i];
+      if (d.radix < 1 || d.which > 2 || !divisorOk(d.div, d.radix)) return false;
+      span[d.which] *= d.radix;
+      logical *= d.radix;
+      if (logical > 0x7fffffffull) return false;  // the decode divides 31-bit numbers
+    }
+    if (span[0] < (uint64_t)tilesM || span[1] < (uint64_t)tilesK || span[2] < (uint64_t)volMbar) return false;
+  } else if (order >= 3) {
     if (superM < 1 || superK < 1) return false;
     logical = (uint64_t)((tilesM + superM - 1) / superM) * ((tilesK + superK - 1) / superK) * superM * superK *
               (uint64_t)volMbar;
@@ -530,6 +522,19 @@ bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk,
     blocks = (uint64_t)xcdChunk * kNumXcd;
   }
   return blocks > 0 && blocks <= 0x7fffffffull && blocks * kTileThreads <= CUTT_HIP_MAX_GRID_LANES;
+}
+
+// The rows of a tile axis over fused ranks: the extents must multiply to the axis' length.
+bool rowRadixOk(const cuttHipRowRadix& rr, int count) {
+  if (rr.n == 0) return true;
+  if (rr.n < 0 || rr.n > CUTT_MAX_TILE_SET) return false;
+  uint64_t vol = 1;
+  for (int k = 0; k < rr.n; k++) {
+    if (rr.extent[k] < 1 || !divisorOk(rr.div[k], rr.extent[k])) return false;
+    vol *= rr.extent[k];
+    if (vol > 0x7fffffffull) return false;
+  }
+  return vol == (uint64_t)count;
 }
 
 // Allow dynamic LDS up to the device limit for a kernel (once per process and kernel).
@@ -610,16 +615,31 @@ hipError_t launchKernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t 
 
 }  // namespace
 
+extern "C" long long cuttHipTiledGrid(const cuttHipTiledArgs* a) {
+  uint64_t blocks = 0;
+  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+    return 0;
+  return (long long)blocks;
+}
+
+extern "C" long long cuttHipTiledCopyGrid(const cuttHipTiledCopyArgs* a) {
+  uint64_t blocks = 0;
+  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+    return 0;
+  return (long long)blocks;
+}
+
 extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || (a->alignedStores != 0 && a->alignedStores != 1) ||
       a->tilesK != (a->volMk + (a->alignedStores ? 128 / a->elemSize - 1 : 0) + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 6 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1) ||
-      (a->alignedStores && a->grouped))
+      a->order < 0 || a->order > 7 || !mbarOk(a->mbar) || (a->grouped != 0 && a->grouped != 1) ||
+      (a->alignedStores && a->grouped) || !rowRadixOk(a->rowsK, a->volMk) || !rowRadixOk(a->rowsM, a->volMm) ||
+      (a->alignedStores && (a->rowsK.n > 0 || a->rowsM.n > 0)))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   return 0;
@@ -628,15 +648,18 @@ extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
 extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, void* out, void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
     return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);
+  const bool fused = a->rowsK.n > 0 || a->rowsM.n > 0;
+#define CUTT_LAUNCH_TILED_F(T, NT, G)                                                                            \
+  (fused ? launchKernel(tiledKernel<T, NT, G, true>, grid, block, 0, s, *a, (const T*)in, (T*)out)               \
+         : launchKernel(tiledKernel<T, NT, G, false>, grid, block, 0, s, *a, (const T*)in, (T*)out))
 #define CUTT_LAUNCH_TILED(T, NT)                                                                        \
   return (int)(a->alignedStores                                                                         \
                    ? launchKernel(tiledAlignedKernel<T, NT>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
-                   : (a->grouped ? launchKernel(tiledKernel<T, NT, true>, grid, block, 0, s, *a, (const T*)in, (T*)out) \
-                                 : launchKernel(tiledKernel<T, NT, false>, grid, block, 0, s, *a, (const T*)in, (T*)out)))
+                   : (a->grouped ? CUTT_LAUNCH_TILED_F(T, NT, true) : CUTT_LAUNCH_TILED_F(T, NT, false)))
 #define CUTT_LAUNCH_TILED_NT(T)                                \
   switch (a->cachePolicy) {                                    \
     case 0: CUTT_LAUNCH_TILED(T, 0);                           \
@@ -650,16 +673,17 @@ extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, voi
   }
 #undef CUTT_LAUNCH_TILED_NT
 #undef CUTT_LAUNCH_TILED
+#undef CUTT_LAUNCH_TILED_F
 }
 
 extern "C" int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* a) {
   if (!a) return (int)hipErrorInvalidValue;
   if ((a->elemSize != 4 && a->elemSize != 8) || a->volMm < 1 || a->volMk < 1 || a->volMbar < 1 ||
       a->tilesM != (a->volMm + kTile - 1) / kTile || a->tilesK != (a->volMk + kTile - 1) / kTile ||
-      a->order < 0 || a->order > 6 || !mbarOk(a->mbar))
+      a->order < 0 || a->order > 7 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   return 0;
@@ -669,7 +693,7 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
                                       void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
     return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);

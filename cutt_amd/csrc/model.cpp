@@ -121,13 +121,25 @@ void mbarOffsets(const cuttHipMbar& mb, uint32_t m, int64_t& offIn, int64_t& off
   }
 }
 
-// One tile of w x h elements (w along rank 0, h along the Mk rank).
+// Offset of row i of a tile axis: i * stride for a single rank, the mixed-radix sum over a fused set.
+inline int64_t rowOffset(const cuttHipRowRadix& rr, int64_t stride, int64_t i) {
+  if (rr.n == 0) return i * stride;
+  int64_t off = 0;
+  for (int k = 0; k < rr.n; k++) {
+    const int64_t e = rr.extent[k];
+    off += (k + 1 < rr.n ? i % e : i) * (int64_t)rr.stride[k];
+    i /= e;
+  }
+  return off;
+}
+
+// One tile of w x h elements (w along the input-contiguous axis, h along the Mk axis).
 Counts tileCost(bool copy, int es, int64_t offIn, int64_t offOut, int64_t m0, int64_t k0, int w, int h,
-                int64_t strideInK, int64_t strideOut) {
+                int64_t strideInK, int64_t strideOut, const cuttHipRowRadix& rowsK, const cuttHipRowRadix& rowsM) {
   Counts c;
   double dummy = 0;
   for (int k = 0; k < h; k++) {
-    runCost(offIn + m0 + (k0 + k) * strideInK, w, es, c.rdLines, c.rdSectors, dummy);
+    runCost(offIn + m0 + rowOffset(rowsK, strideInK, k0 + k), w, es, c.rdLines, c.rdSectors, dummy);
     c.rdInstr += 1;
   }
   if (copy) {
@@ -137,7 +149,7 @@ Counts tileCost(bool copy, int es, int64_t offIn, int64_t offOut, int64_t m0, in
     }
   } else {
     for (int m = 0; m < w; m++) {
-      runCost(offOut + k0 + (m0 + m) * strideOut, h, es, c.wrLines, c.wrSectors, c.wrPartial);
+      runCost(offOut + k0 + rowOffset(rowsM, strideOut, m0 + m), h, es, c.wrLines, c.wrSectors, c.wrPartial);
       c.wrInstr += 1;
     }
     // LDS: one padded-tile write and one read per element row, conflict free.
@@ -146,26 +158,59 @@ Counts tileCost(bool copy, int es, int64_t offIn, int64_t offOut, int64_t m0, in
   return c;
 }
 
-Counts tiledSample(const Plan& p, bool copy, uint32_t m) {
+Counts tiledSample(const Plan& p, bool copy, uint32_t m, std::minstd_rand0& rng, bool everyTile) {
   const int es = p.pb.elemSize;
   const int volMm = copy ? p.tcopy.volMm : p.tiled.volMm;
   const int volMk = copy ? p.tcopy.volMk : p.tiled.volMk;
   const int64_t sIn = copy ? p.tcopy.strideInK : p.tiled.strideInK;
   const int64_t sOut = copy ? p.tcopy.strideOutK : p.tiled.strideOutM;
+  static const cuttHipRowRadix kSingle = {};
+  const cuttHipRowRadix& rowsK = copy ? kSingle : p.tiled.rowsK;
+  const cuttHipRowRadix& rowsM = copy ? kSingle : p.tiled.rowsM;
   int64_t offIn, offOut;
   mbarOffsets(copy ? p.tcopy.mbar : p.tiled.mbar, m, offIn, offOut);
   const int fullM = volMm / kTile, fullK = volMk / kTile;
   const int remM = volMm % kTile, remK = volMk % kTile;
   Counts total;
-  if (fullM && fullK)
-    total.add(tileCost(copy, es, offIn, offOut, 0, 0, kTile, kTile, sIn, sOut), (double)fullM * fullK);
-  if (remM && fullK)
-    total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, 0, remM, kTile, sIn, sOut), fullK);
-  if (remK && fullM)
-    total.add(tileCost(copy, es, offIn, offOut, 0, (int64_t)fullK * kTile, kTile, remK, sIn, sOut), fullM);
-  if (remM && remK)
-    total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, (int64_t)fullK * kTile, remM, remK,
-                       sIn, sOut), 1);
+  if (rowsK.n == 0 && rowsM.n == 0) {
+    // equally spaced rows: the full tiles of one Mbar position all cost the same
+    if (fullM && fullK)
+      total.add(tileCost(copy, es, offIn, offOut, 0, 0, kTile, kTile, sIn, sOut, rowsK, rowsM), (double)fullM * fullK);
+    if (remM && fullK)
+      total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, 0, remM, kTile, sIn, sOut, rowsK, rowsM), fullK);
+    if (remK && fullM)
+      total.add(tileCost(copy, es, offIn, offOut, 0, (int64_t)fullK * kTile, kTile, remK, sIn, sOut, rowsK, rowsM), fullM);
+    if (remM && remK)
+      total.add(tileCost(copy, es, offIn, offOut, (int64_t)fullM * kTile, (int64_t)fullK * kTile, remM, remK,
+                         sIn, sOut, rowsK, rowsM), 1);
+    return total;
+  }
+  // Rows over fused ranks start at offsets that differ from tile to tile: a few tiles of every kind
+  // (inner, last along Mm, last along Mk, corner) are walked and stand for the others (all of them
+  // when the caller asks for the exact count).
+  const int tilesM = fullM + (remM ? 1 : 0), tilesK = fullK + (remK ? 1 : 0);
+  auto sample = [&](int tmLo, int tmHi, int tkLo, int tkHi) {  // tiles [tmLo, tmHi) x [tkLo, tkHi)
+    const int64_t count = (int64_t)(tmHi - tmLo) * (tkHi - tkLo);
+    if (count <= 0) return;
+    const int64_t n = everyTile ? count : std::min<int64_t>(count, 6);
+    for (int64_t i = 0; i < n; i++) {
+      int tm, tk;
+      if (n == count) {
+        tm = tmLo + (int)(i % (tmHi - tmLo));
+        tk = tkLo + (int)(i / (tmHi - tmLo));
+      } else {
+        tm = tmLo + (int)(rng() % (uint32_t)(tmHi - tmLo));
+        tk = tkLo + (int)(rng() % (uint32_t)(tkHi - tkLo));
+      }
+      const int w = std::min(kTile, volMm - tm * kTile), h = std::min(kTile, volMk - tk * kTile);
+      total.add(tileCost(copy, es, offIn, offOut, (int64_t)tm * kTile, (int64_t)tk * kTile, w, h, sIn, sOut, rowsK, rowsM),
+                (double)count / n);
+    }
+  };
+  sample(0, fullM, 0, fullK);
+  sample(fullM, tilesM, 0, fullK);
+  sample(0, fullM, fullK, tilesK);
+  sample(fullM, tilesM, fullK, tilesK);
   return total;
 }
 
@@ -257,7 +302,7 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     std::uniform_int_distribution<uint32_t> pick(0, volMbar - 1);
     for (int i = 0; i < ns; i++) {
       const uint32_t m = ((uint32_t)ns == volMbar) ? (uint32_t)i : pick(rng);
-      total.add(tiledSample(plan, copy, m), (double)volMbar / ns);
+      total.add(tiledSample(plan, copy, m, rng, numSamples == 0), (double)volMbar / ns);
     }
   } else {
     if (!plan.buildTables()) return false;
@@ -360,11 +405,13 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
       return 0.0;
     };
     // input runs lie along rank 0; output runs along the first output rank (Tiled) or rank 0 (TiledCopy)
-    r.rdEdgeDist = tilesM > 1 ? 1.0 : (pb.rank > 1 ? mbarDist(1, true) : 0.0);
+    // (a Tiled plan over fused rank sets: the runs end where the set ends)
+    const int nextIn = copy ? 1 : plan.split.numMm, nextOut = copy ? 1 : plan.split.numMk;
+    r.rdEdgeDist = tilesM > 1 ? 1.0 : (nextIn < pb.rank ? mbarDist(nextIn, true) : 0.0);
     if (copy) {
       r.wrEdgeDist = tilesM > 1 ? 1.0 : (pb.rank > 1 ? mbarDist(pb.perm[1], false) : 0.0);
     } else {
-      r.wrEdgeDist = tilesK > 1 ? std::min(superM, tilesM) : (pb.rank > 1 ? mbarDist(pb.perm[1], false) : 0.0);
+      r.wrEdgeDist = tilesK > 1 ? std::min(superM, tilesM) : (nextOut < pb.rank ? mbarDist(pb.perm[nextOut], false) : 0.0);
     }
   }
 

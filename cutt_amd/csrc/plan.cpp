@@ -555,9 +555,67 @@ struct TileOrdering {
   uint32_t xcdChunk, superM, superK;
 };
 
+// Order 7: the digits of `text` ("m2,k8,b0,m0,k0": coordinate letter + radix, fastest first; radix 0 = what
+// is left of the coordinate).  A coordinate whose digits do not reach its extent gets one more, slowest,
+// digit.  Returns the number of logical workgroups, 0 if the text is malformed.
+int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK, int64_t volMbar, cuttHipTileDigits& dg) {
+  std::memset(&dg, 0, sizeof(dg));
+  const int64_t extent[3] = {tilesM, tilesK, volMbar};
+  int64_t span[3] = {1, 1, 1};
+  auto push = [&](int which, int64_t radix) {
+    if (dg.n >= CUTT_MAX_TILE_DIGITS || radix < 1 || radix > 0x7fffffffll) return false;
+    if (radix == 1) return true;
+    dg.d[dg.n].which = (uint32_t)which;
+    dg.d[dg.n].radix = (uint32_t)radix;
+    dg.d[dg.n].div = cuttHipMakeDivisor((uint32_t)radix);
+    dg.n++;
+    span[which] *= radix;
+    return true;
+  };
+  size_t pos = 0;
+  while (pos < text.size()) {
+    const char c = text[pos++];
+    const int which = c == 'm' ? 0 : (c == 'k' ? 1 : (c == 'b' ? 2 : -1));
+    if (which < 0) return 0;
+    int64_t radix = 0;
+    while (pos < text.size() && text[pos] >= '0' && text[pos] <= '9') radix = radix * 10 + (text[pos++] - '0');
+    if (pos < text.size() && text[pos] == ',') pos++;
+    if (radix == 0) radix = ceilDiv(extent[which], span[which]);
+    if (!push(which, radix)) return 0;
+  }
+  for (int w : {2, 0, 1})
+    if (span[w] < extent[w] && !push(w, ceilDiv(extent[w], span[w]))) return 0;
+  if (dg.n == 0) {  // a single workgroup
+    dg.d[0].which = 0; dg.d[0].radix = 1; dg.d[0].div = cuttHipMakeDivisor(1); dg.n = 1;
+  }
+  int64_t logical = 1;
+  for (int i = 0; i < dg.n; i++) {
+    logical *= dg.d[i].radix;
+    if (logical > 0x7fffffffll) return 0;
+  }
+  return logical;
+}
+
 int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
                     int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, bool mbarBetween,
-                    bool beyondCache, TileOrdering& o) {
+                    bool beyondCache, TileOrdering& o, cuttHipTileDigits& dg) {
+  std::memset(&dg, 0, sizeof(dg));
+  if (!opt.tileDigits.empty()) {
+    const int64_t logical = parseTileDigits(opt.tileDigits, tilesM, tilesK, volMbar, dg);
+    if (logical > 0) {
+      o.order = 7;
+      o.superM = o.superK = 1;
+      o.xcdChunk = 0;
+      if (opt.xcdAware && logical >= 64) {
+        const int64_t chunk = ceilDiv(logical, kNumXcd);
+        if (chunk * kNumXcd <= 0x7fffffffll) {
+          o.xcdChunk = (uint32_t)chunk;
+          return chunk * kNumXcd;
+        }
+      }
+      return logical;
+    }
+  }
   // Default: strips of super-tiles, each strip visited for all Mbar positions in turn (order 5;
   // with one Mbar position that is order 3).  The runs of consecutive Mbar positions are usually
   // neighbours in memory, so their shared lines meet in the L2: against finishing one Mbar position
@@ -661,8 +719,27 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.volMk = (int)sp.volMk;
     a.strideInK = (uint32_t)pb.strideIn[rk];
     a.strideOutM = (uint32_t)pb.strideOut[0];
+    // A tile axis over several fused ranks: the rows' offsets follow the ranks' extents and strides.
+    if (sp.numMm > CUTT_MAX_TILE_SET || sp.numMk > CUTT_MAX_TILE_SET || sp.volMm > 0x7fffffffll || sp.volMk > 0x7fffffffll)
+      return false;
+    if (sp.numMk > 1) {
+      a.rowsK.n = sp.numMk;
+      for (int j = 0; j < sp.numMk; j++) {
+        a.rowsK.extent[j] = (uint32_t)pb.dim[pb.perm[j]];
+        a.rowsK.stride[j] = (uint32_t)pb.strideIn[pb.perm[j]];
+        a.rowsK.div[j] = cuttHipMakeDivisor(a.rowsK.extent[j]);
+      }
+    }
+    if (sp.numMm > 1) {
+      a.rowsM.n = sp.numMm;
+      for (int r = 0; r < sp.numMm; r++) {
+        a.rowsM.extent[r] = (uint32_t)pb.dim[r];
+        a.rowsM.stride[r] = (uint32_t)pb.strideOut[r];
+        a.rowsM.div[r] = cuttHipMakeDivisor(a.rowsM.extent[r]);
+      }
+    }
     a.tilesM = (int)tilesM;
-    a.alignedStores = opt.tiledAligned > 0 ? 1 : 0;
+    a.alignedStores = opt.tiledAligned > 0 && sp.numMm == 1 && sp.numMk == 1 ? 1 : 0;
     a.tilesK = (int)ceilDiv(sp.volMk + (a.alignedStores ? 128 / pb.elemSize - 1 : 0), kTile);
     a.volMbar = (int)sp.volMbar;
     TileOrdering o;
@@ -674,7 +751,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
     const bool beyondCache = (double)pb.volume * pb.elemSize > 0.75 * cacheBytes;
     plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
-                                 sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o);
+                                 sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o, a.digits);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     a.grouped = opt.tiledGrouped > 0 && !a.alignedStores ? 1 : 0;  // -1: decided from the model's estimate later
@@ -695,7 +772,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     PlannerOptions copt = opt;
     copt.superAuto = false;  // (the measured exceptions are for the Tiled kernel only)
-    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, o);
+    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, o, a.digits);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
@@ -745,21 +822,48 @@ void addTrivial(const Problem& red, const PlannerOptions& opt, std::vector<Plan>
 void addTiled(const Problem& red, const cuttHipDeviceProps& props, const PlannerOptions& opt,
               std::vector<Plan>& plans) {
   if (red.rank < 2) return;
-  Plan p;
-  p.pb = red;
-  p.fromReduced = true;
-  if (red.perm[0] != 0) {
-    // The leading rank moves: 2-D tiles between input rank 0 and the rank that leads the output.
-    p.method = p.split.method = kTiled;
-    p.split.update(1, 1, red);
-  } else {
+  if (red.perm[0] == 0) {
     // The leading rank stays: copy rows, tile over the second output rank.
+    Plan p;
+    p.pb = red;
+    p.fromReduced = true;
     p.method = p.split.method = kTiledCopy;
     p.split.update(1, 2, red);
+    if (!allowed(opt, p.method)) return;
+    if (!setupTiled(p, props, opt)) return;
+    if (!exists(p.split, plans)) plans.push_back(std::move(p));
+    return;
   }
-  if (!allowed(opt, p.method)) return;
-  if (!setupTiled(p, props, opt)) return;
-  if (!exists(p.split, plans)) plans.push_back(std::move(p));
+  if (!allowed(opt, kTiled)) return;
+  // The leading rank moves: 2-D tiles between the ranks that lead the input (Mm) and the ranks that
+  // lead the output (Mk).  One rank on each side is the reference's Tiled method
+  // (src/cuttplan.cpp:494-511); here either side may also run over its first two, three or four
+  // ranks fused - the first numMm input ranks are one contiguous run of the input, the first numMk
+  // output ranks one of the output, as long as the two sets share no rank - which the reference lists
+  // as future work (README.md:197-199).  A short leading rank (36 or 166 elements) then no longer
+  // leaves the 64-wide tiles half empty or cuts every row into a long and a short piece.  A side is
+  // extended only while what it has so far is short (below 2048 elements, 32 tiles) and not a whole
+  // number of tiles: otherwise its tiles are full anyway.
+  constexpr int64_t kFuseBelow = 2048;
+  const int maxSet = opt.tiledFuse == 0 ? 1 : CUTT_MAX_TILE_SET;
+  int64_t volM = 1;
+  for (int numMm = 1; numMm <= maxSet && numMm < red.rank; numMm++) {
+    if (numMm > 1 && (volM >= kFuseBelow || volM % kTile == 0 || red.gapIn[numMm - 2])) break;
+    volM *= red.dim[numMm - 1];
+    int64_t volK = 1;
+    for (int numMk = 1; numMk <= maxSet && numMm + numMk <= red.rank; numMk++) {
+      if (numMk > 1 && (volK >= kFuseBelow || volK % kTile == 0 || red.gapOut[red.perm[numMk - 2]])) break;
+      if (red.perm[numMk - 1] < numMm) break;  // the sets would share a rank (and so would every larger Mk)
+      volK *= red.dim[red.perm[numMk - 1]];
+      Plan p;
+      p.pb = red;
+      p.fromReduced = true;
+      p.method = p.split.method = kTiled;
+      p.split.update(numMm, numMk, red);
+      if (!setupTiled(p, props, opt)) continue;
+      if (!exists(p.split, plans)) plans.push_back(std::move(p));
+    }
+  }
 }
 
 void addPacked(const Problem& pb, bool fromReduced, const cuttHipDeviceProps& props,

@@ -147,6 +147,9 @@ struct PlannerOptions {
   int tiledOrder = -1;      // -1 = planner's choice (super-tiles)
   int superM = 8, superK = 4096;  // super-tile shape for tiled orders 3-6: strips of 8 tiles along Mm
   bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
+  std::string tileDigits;   // non-empty: tiled order 7 with this mixed-radix numbering, fastest digit first, e.g.
+                            // "m2,k8,b0,m0,k0" (m / k = tile along Mm / Mk, b = Mbar position; radix 0 = what is left)
+  int tiledFuse = -1;       // Tiled over fused rank sets: -1 = planner's choice, 0 = one rank per side only
   int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time
   int elemsPerThread = 0;    // Packed/PackedSplit: 0 = planner's choice, else 1, 2, 4, 8 or 16

@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 
 #include "hip_layer.h"
+#include "mbar_decode.h"
 
 namespace cutt {
 
@@ -36,11 +37,14 @@ constexpr int kWaves = kTileThreads / 64;
 // different columns at any one time, and with small patches their reads and their writes both spread over
 // the address space (measured on C2: 2 x 2 patches 5.3 TB/s in order 5, 6.15 TB/s in order 6; which shapes
 // gain is not predictable from the strides, so only the measuring planner uses it).
+// Order 7 reads the logical index as a mixed-radix number whose digits are dealt out to the three
+// coordinates (cuttHipTileDigits): any nesting of patches, strips and Mbar runs can be written that way.
 constexpr uint32_t kNumXcd = 8;
 
 struct TileOrder {
   int order;
   uint32_t xcdChunk, superM, superK;
+  const cuttHipTileDigits* digits;  // order 7 (points into the kernel arguments)
 };
 
 __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint32_t tilesM,
@@ -65,6 +69,21 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
     m = t / tilesM;
     tm = t - m * tilesM;
     return m < volMbar;
+  } else if (o.order == 7) {
+    const cuttHipTileDigits& dg = *o.digits;
+    uint32_t c0 = 0, c1 = 0, c2 = 0, w0 = 1, w1 = 1, w2 = 1, rest = l;
+    for (int i = 0; i < dg.n; i++) {
+      const cuttHipTileDigit d = dg.d[i];
+      const uint32_t q = fastDivide(rest, d.div.mul, d.div.shift, d.div.add);
+      // the slowest digit takes what is left (beyond its radix on the padding workgroups)
+      const uint32_t v = i + 1 < dg.n ? rest - q * d.radix : rest;
+      rest = q;
+      if (d.which == 0) { c0 += v * w0; w0 *= d.radix; }
+      else if (d.which == 1) { c1 += v * w1; w1 *= d.radix; }
+      else { c2 += v * w2; w2 *= d.radix; }
+    }
+    tm = c0; tk = c1; m = c2;
+    return tm < tilesM && tk < tilesK && m < volMbar;
   }
   const uint32_t nSuperM = (tilesM + o.superM - 1) / o.superM, nSuperK = (tilesK + o.superK - 1) / o.superK;
   const uint32_t per = o.superM * o.superK;
@@ -91,6 +110,91 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
     tm = (st / nSuperK) * o.superM + (w / o.superK);
   }
   return m < volMbar && tm < tilesM && tk < tilesK;
+}
+
+// Offset of row `i` of a tile axis that runs over the fused ranks of `rr` (rr.n >= 1), per lane.
+__device__ __forceinline__ uint32_t rowOffset(const cuttHipRowRadix& rr, uint32_t i) {
+  uint32_t off = 0;
+  for (int k = 0; k + 1 < rr.n; k++) {
+    const uint32_t q = fastDivide(i, rr.div[k].mul, rr.div[k].shift, rr.div[k].add);
+    off += (i - q * rr.extent[k]) * rr.stride[k];
+    i = q;
+  }
+  return off + i * rr.stride[rr.n - 1];
+}
+
+// The offsets of the 64 rows of a tile that starts at row `first` of an axis with `count` rows, one
+// row per lane (rows beyond the axis repeat the last one); `stride` is used when the axis is a single rank.
+__device__ __forceinline__ uint32_t tileRowOffsets(const cuttHipRowRadix& rr, uint32_t stride, uint32_t first,
+                                                   uint32_t count, uint32_t lane) {
+  const uint32_t i = min(first + lane, count - 1);
+  return rr.n > 0 ? rowOffset(rr, i) : i * stride;
+}
+
+// What a lane of a Tiled workgroup needs to address the rows of its tile; shared by the transpose
+// kernel and the kernel that replays its address stream.
+struct TileLanes {
+  uint32_t m0, k0;            // first element of the tile along Mm / Mk
+  uint32_t wM, wK;            // last valid column / row inside the tile (edge tiles are narrower)
+  uint32_t groupsM, groupsK;  // groups of 16 rows that hold valid rows, per side
+  uint32_t cx, ck;            // the lane's (clamped) position along Mm when reading, along Mk when writing
+  uint32_t rdBase, wrBase;    // element offset of the lane's column in row 0 of the tile's axis origin
+  uint32_t rowK, rowM, waveU; // FUSED: row offsets held one per lane, and the wave index as a scalar
+};
+
+template <bool FUSED>
+__device__ __forceinline__ TileLanes tileLanes(const cuttHipTiledArgs& a, uint32_t tm, uint32_t tk, uint32_t offIn,
+                                               uint32_t offOut, uint32_t lane, uint32_t wave) {
+  TileLanes t;
+  t.m0 = tm * kTile;
+  t.k0 = tk * kTile;
+  // Edge tiles are handled without branches: indices are clamped to the last valid row / column,
+  // so out-of-range lanes repeat the access of the edge element (same address, same value).  That
+  // keeps the loop bodies straight-line code, and all 16 loads of a lane go out back to back.
+  t.wM = min((uint32_t)kTile, (uint32_t)a.volMm - t.m0) - 1;
+  t.wK = min((uint32_t)kTile, (uint32_t)a.volMk - t.k0) - 1;
+  // The 16 rows of a lane come in kRowGroups groups of 4; group g covers tile rows 16g..16g+15
+  // over the four waves.  An edge tile skips the groups that lie entirely beyond its valid part
+  // (a test that is uniform over the workgroup), so that a thin edge costs a quarter of a tile's
+  // instructions, not all of them; inside a group the clamping above still applies.
+  t.groupsK = (t.wK >> 4) + 1;
+  t.groupsM = (t.wM >> 4) + 1;
+  t.cx = min(lane, t.wM);
+  t.ck = min(lane, t.wK);
+  t.rdBase = offIn + t.m0 + t.cx;
+  t.wrBase = offOut + t.k0 + t.ck;
+  t.rowK = t.rowM = t.waveU = 0;
+  if constexpr (FUSED) {
+    // lane l holds the input offset of row k0 + l along Mk and the output offset of row m0 + l along
+    // Mm; the row a wave asks for is wave-uniform
+    t.rowK = tileRowOffsets(a.rowsK, a.strideInK, t.k0, (uint32_t)a.volMk, lane);
+    t.rowM = tileRowOffsets(a.rowsM, a.strideOutM, t.m0, (uint32_t)a.volMm, lane);
+    t.waveU = (uint32_t)__builtin_amdgcn_readfirstlane((int)wave);
+  }
+  return t;
+}
+
+// Element offset of the lane's j-th load (row wave + 4 j of the tile, clamped) / store.
+template <bool FUSED>
+__device__ __forceinline__ uint32_t tileReadElem(const TileLanes& t, const cuttHipTiledArgs& a, uint32_t wave, int j) {
+  if constexpr (FUSED) {
+    const uint32_t r = min(t.waveU + kWaves * j, t.wK);
+    return t.rdBase + (uint32_t)__builtin_amdgcn_readlane((int)t.rowK, (int)r);
+  } else {
+    const uint32_t r = min(wave + kWaves * j, t.wK);
+    return t.rdBase + (t.k0 + r) * a.strideInK;
+  }
+}
+
+template <bool FUSED>
+__device__ __forceinline__ uint32_t tileWriteElem(const TileLanes& t, const cuttHipTiledArgs& a, uint32_t wave, int j) {
+  if constexpr (FUSED) {
+    const uint32_t r = min(t.waveU + kWaves * j, t.wM);
+    return t.wrBase + (uint32_t)__builtin_amdgcn_readlane((int)t.rowM, (int)r);
+  } else {
+    const uint32_t r = min(wave + kWaves * j, t.wM);
+    return t.wrBase + (t.m0 + r) * a.strideOutM;
+  }
 }
 
 }  // namespace cutt

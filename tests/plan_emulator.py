@@ -25,7 +25,7 @@ def _mbar_offsets(tab, vol_mbar):
     return off_in, off_out
 
 
-def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k):
+def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k, digits=()):
     """The kernels' workgroup-index decoding visits every (tile, Mbar position) exactly once."""
     b = np.arange(num_blocks, dtype=np.int64)
     if xcd_chunk:
@@ -33,7 +33,24 @@ def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk,
         l = (b % 8) * xcd_chunk + b // 8
     else:
         l = b
-    if order == 0:
+    if order == 7:
+        # mixed-radix number, fastest digit first; every digit belongs to one coordinate
+        n = len(digits) // 2
+        assert 1 <= n <= 12
+        coord = [np.zeros_like(l), np.zeros_like(l), np.zeros_like(l)]
+        weight = [1, 1, 1]
+        rest = l.copy()
+        for i in range(n):
+            which, radix = int(digits[2 * i]), int(digits[2 * i + 1])
+            assert which in (0, 1, 2) and radix >= 1
+            v = rest % radix if i + 1 < n else rest
+            rest = rest // radix
+            coord[which] = coord[which] + v * weight[which]
+            weight[which] *= radix
+        assert weight[0] >= tiles_m and weight[1] >= tiles_k and weight[2] >= vol_mbar
+        tm, tk, m = coord
+        ok = (tm < tiles_m) & (tk < tiles_k) & (m < vol_mbar)
+    elif order == 0:
         t, m = l // vol_mbar, l % vol_mbar
         tk, tm = t // tiles_m, t % tiles_m
         ok = tk < tiles_k
@@ -93,14 +110,34 @@ def emulate(cands, idx, data):
     if name in ("Tiled", "TiledCopy"):
         vol_mm, vol_mk, s_in_k, s_out, tiles_m, tiles_k, vol_mbar, order, xcd_chunk, sup_m, sup_k = [int(v) for v in cands.data(idx, 1)]
         assert tiles_m == -(-vol_mm // 64) and tiles_k == -(-vol_mk // 64)
-        _check_tile_decode(info.numBlocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k)
+        _check_tile_decode(info.numBlocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk, sup_m, sup_k,
+                           cands.data(idx, 8) if order == 7 else ())
         off_in, off_out = _mbar_offsets(mbar, vol_mbar)
         x = np.arange(vol_mm, dtype=np.int64)
         k = np.arange(vol_mk, dtype=np.int64)
+
+        def row_offsets(i, radix, stride):
+            """Offsets of the rows of a tile axis: i * stride, or the mixed-radix sum over a fused rank set."""
+            if len(radix) == 0:
+                return i * stride
+            n = len(radix) // 2
+            assert n <= 4 and int(np.prod([int(radix[2 * j]) for j in range(n)])) == i.size
+            off = np.zeros_like(i)
+            rest = i.copy()
+            for j in range(n):
+                e, st = int(radix[2 * j]), int(radix[2 * j + 1])
+                off += (rest % e if j + 1 < n else rest) * st
+                rest //= e
+            return off
+
+        rows_k = cands.data(idx, 7, 0) if name == "Tiled" else ()
+        rows_m = cands.data(idx, 7, 1) if name == "Tiled" else ()
         xx, kk = np.meshgrid(x, k, indexing="ij")
-        src = (xx + kk * s_in_k).ravel()
+        in_k = row_offsets(k, rows_k, s_in_k)
+        src = (xx + in_k[None, :]).ravel()
         if name == "Tiled":
-            dst = (kk + xx * s_out).ravel()
+            out_m = row_offsets(x, rows_m, s_out)
+            dst = (kk + out_m[:, None]).ravel()
         else:
             dst = (xx + kk * s_out).ravel()
         for m in range(vol_mbar):

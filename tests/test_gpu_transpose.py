@@ -620,3 +620,55 @@ def test_tile_orders_and_patch_shapes_of_the_tiled_kernels(gpu, monkeypatch):
                         seen.add((info.method_name, order))
         say("tile orders dim=%s perm=%s done" % (dim, perm))
     assert {("Tiled", o) for o in range(7)} <= seen and {("TiledCopy", o) for o in range(7)} <= seen
+
+
+def test_tiled_over_fused_rank_sets(gpu):
+    """Tiled candidates whose tile axes run over two to four fused ranks (the reference's README.md:197-199 lists
+    them as future work): every candidate of shapes with short or ragged leading ranks on either side, both
+    widths, against the oracle; and the device's count of the address stream against the host model's."""
+    import cutt_amd as cutt
+    cases = [((36, 50, 1000, 11), (2, 0, 3, 1)), ((7, 9, 11, 700, 5), (3, 1, 0, 4, 2)), ((700, 9, 36, 5, 11), (2, 3, 0, 4, 1)),
+             ((6, 11, 50, 7, 13), (4, 3, 2, 1, 0)), ((3, 5, 7, 40, 9, 11), (5, 4, 3, 1, 0, 2)), ((166, 3, 500, 41), (2, 0, 3, 1)),
+             ((100, 2, 3, 2, 90, 2, 3, 2), (4, 5, 6, 7, 3, 2, 1, 0))]
+    sets = set()
+    st = gpu.stream_handle()
+    for dim, perm in cases:
+        for es in (4, 8):
+            data = gpu.seeded(int(np.prod(dim)), es, seed=es + len(dim))
+            with cutt.Candidates(dim, perm, es) as c:
+                idx = [i for i in range(len(c)) if c.info(i).method_name == "Tiled"]
+            for i in idx:
+                say("fused Tiled candidate %d dim=%s perm=%s es=%d" % (i, dim, perm, es))
+                info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i)
+                sets.add((info.numMm, info.numMk))
+                if info.numMm > 1 or info.numMk > 1:
+                    rc, h = cutt.cuttPlanFromCandidate(len(dim), list(dim), list(perm), es, st, i)
+                    assert rc == cutt.CUTT_SUCCESS
+                    dev, mod = cutt.count_address_stream(h, 0)
+                    d, m = dev.as_dict(), mod.as_dict()
+                    for k in ("rdInstr", "wrInstr", "rdLines", "wrLines", "rdSectors", "wrSectors", "wrPartialLines"):
+                        assert d[k] == m[k], (dim, perm, es, k, d[k], m[k])
+                    cutt.cuttDestroy(h)
+    assert {(2, 1), (1, 2), (2, 2), (3, 1), (4, 1)} <= sets, sets
+
+
+def test_free_tile_numbering(gpu, monkeypatch):
+    """Tile order 7 (the workgroup index as a mixed-radix number whose digits are dealt out to the two tile
+    coordinates and the Mbar position) on shapes with edge tiles, for Tiled and TiledCopy, both widths."""
+    import cutt_amd as cutt
+    import oracle
+    cases = [((200, 6, 300, 3), (2, 1, 0, 3)), ((70, 130), (1, 0)), ((650, 3, 5, 70), (3, 1, 2, 0)), ((150, 7, 300), (0, 2, 1)),
+             ((512, 12, 512, 3), (2, 1, 0, 3))]
+    for dim, perm in cases:
+        for es in (4, 8):
+            data = gpu.seeded(int(np.prod(dim)), es, seed=3 + es)
+            expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
+            for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0"]:
+                monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
+                with cutt.Candidates(dim, perm, es) as c:
+                    idx = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]
+                assert idx
+                for i in idx:
+                    info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
+                    assert info.tiledOrder == 7
+        say("tile digits dim=%s perm=%s done" % (dim, perm))

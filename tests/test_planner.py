@@ -185,7 +185,7 @@ def test_plans_do_not_depend_on_the_number_of_planner_threads(cutt, monkeypatch)
 def test_rows_in_groups_only_for_large_unaligned_tensors_of_4_byte_elements(cutt):
     def tiled(dim, perm, es):
         infos, best = method_set(cutt, dim, perm, es)
-        t = [i for i in infos if i.method_name == "Tiled"]
+        t = [i for i in infos if i.method_name == "Tiled" and i.numMm == 1 and i.numMk == 1]  # one rank per side
         assert len(t) == 1
         return t[0].tiledGrouped
     assert tiled((4457, 44570), (1, 0), 4) == 1          # rows of 17828 bytes, 795 MB
@@ -200,7 +200,7 @@ def test_rows_in_groups_only_for_large_unaligned_tensors_of_4_byte_elements(cutt
 def test_super_tile_shapes_of_the_tiled_plan(cutt):
     def tiled(dim, perm, es):
         infos, best = method_set(cutt, dim, perm, es)
-        t = [i for i in infos if i.method_name == "Tiled"]
+        t = [i for i in infos if i.method_name == "Tiled" and i.numMm == 1 and i.numMk == 1]
         assert len(t) == 1
         return t[0].tiledOrder, t[0].superM, t[0].superK
     # strips of 8 tiles through all of Mk, every strip for all Mbar positions in turn
@@ -263,3 +263,50 @@ def test_random_shapes_every_candidate(cutt, oracle_mod):
         seen |= check_all_candidates(cutt, oracle_mod, dim, perm, es, lds=lds)
         done += 1
     assert {"Tiled", "TiledCopy", "Packed", "PackedSplit"} <= seen
+
+
+def test_tiled_over_fused_rank_sets(cutt, oracle_mod):
+    # Mm = the first ranks of the input, Mk = the first ranks of the output, each a contiguous run of
+    # its side (the reference's README.md:197-199 lists this as future work).  Every such candidate is
+    # replayed against the oracle; the candidate lists must hold tiles over two and three fused ranks.
+    sets = set()
+    for dim, perm in [((36, 5, 70, 9), (2, 3, 0, 1)),        # Mm = {0, 1}: 180 elements
+                      ((7, 9, 11, 70), (3, 1, 0, 2)),         # Mm = {0, 1, 2}: 693
+                      ((70, 9, 36, 5), (2, 3, 0, 1)),         # Mk = {2, 3}: 180
+                      ((6, 11, 5, 7, 13), (4, 3, 2, 1, 0)),   # both sides: Mm = {0, 1}, Mk = {4, 3}
+                      ((3, 5, 7, 4, 9, 11), (5, 4, 3, 1, 0, 2)),
+                      ((166, 3, 50, 4), (2, 0, 3, 1))]:       # Mm stops at rank 0: rank 1 is not next to it in Mk's way
+        for es in (4, 8):
+            check_all_candidates(cutt, oracle_mod, dim, perm, es, need="Tiled")
+            with cutt.Candidates(dim, perm, es) as c:
+                for i in range(len(c)):
+                    info = c.info(i)
+                    if info.method_name == "Tiled":
+                        sets.add((info.numMm, info.numMk))
+                        # the two sets never share a rank
+                        assert info.volMm * info.volMk * info.volMbar == int(np.prod(dim))
+    assert (2, 1) in sets and (1, 2) in sets and (2, 2) in sets and (3, 1) in sets, sets
+
+
+def test_fused_tiled_sets_only_where_tiles_would_be_ragged(cutt):
+    # a leading rank that is a whole number of tiles is not extended
+    infos, best = method_set(cutt, (1024, 64, 1024, 3), (2, 1, 0, 3), 8)
+    assert [(i.numMm, i.numMk) for i in infos if i.method_name == "Tiled"] == [(1, 1)]
+    infos, best = method_set(cutt, (36, 50, 1000, 111), (2, 0, 3, 1), 8)
+    assert {(i.numMm, i.numMk) for i in infos if i.method_name == "Tiled"} >= {(1, 1), (2, 1)}
+
+
+def test_free_tile_numbering(cutt, oracle_mod, monkeypatch):
+    # tile order 7: the workgroup index as a mixed-radix number whose digits are dealt out to the tile
+    # along Mm, the tile along Mk and the Mbar position; every tile must be visited exactly once
+    cutt.set_method_override(4)  # Tiled only
+    try:
+        for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0"]:
+            monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
+            for dim, perm in [((200, 6, 300, 3), (2, 1, 0, 3)), ((70, 130), (1, 0)), ((650, 3, 5, 70), (3, 1, 2, 0))]:
+                with cutt.Candidates(dim, perm, 8) as c:
+                    orders = [c.info(i).tiledOrder for i in range(len(c)) if c.info(i).method_name == "Tiled"]
+                    assert orders and all(o == 7 for o in orders), (digits, dim, orders)
+                check_all_candidates(cutt, oracle_mod, dim, perm, 8, need="Tiled")
+    finally:
+        cutt.set_method_override(0)
