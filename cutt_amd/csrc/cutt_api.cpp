@@ -86,7 +86,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_TILED_FUSE"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
@@ -417,6 +417,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_TILED_ALIGNED")) opt.tiledAligned = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILE_DIGITS")) opt.tileDigits = e;
   if (const char* e = std::getenv("CUTT_TILED_FUSE")) opt.tiledFuse = std::atoi(e) != 0 ? 1 : 0;
+  if (const char* e = std::getenv("CUTT_ADDRESS_BITS")) opt.addressBits = std::atoi(e) != 0;
   return opt;
 }
 
@@ -743,6 +744,10 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
       cur.superM = (int)(t ? plans[best].tiled.superM : plans[best].tcopy.superM);
       cur.superK = (int)(t ? plans[best].tiled.superK : plans[best].tcopy.superK);
       cur.superAuto = false;
+      if (cur.tiledOrder == 7) {  // a free numbering is reproduced from its digits
+        cur.tileDigits = formatTileDigits(t ? plans[best].tiled.digits : plans[best].tcopy.digits);
+        cur.tiledOrder = -1;
+      }
     } else {
       cur.maxItemsPerBlock = plans[best].packed.itemsPerBlock;
       cur.itemOrder = plans[best].packed.itemOrder;
@@ -788,6 +793,7 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
         if (k.order == start.tiledOrder && k.superM == start.superM && k.superK == start.superK) continue;
         PlannerOptions v = cur;
         v.tiledOrder = k.order; v.superM = k.superM; v.superK = k.superK;
+        v.tileDigits.clear();
         if (tryVariant(v, false)) cur = v;
       }
       // sixteen or four rows per lane in flight
@@ -1215,13 +1221,14 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
         }
       }
       break;
-    case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix) of the digits, fastest first
+    case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix, weight) of the digits, fastest first
       if (p.method != kTiled && p.method != kTiledCopy) return -1;
       {
         const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
         for (int k = 0; k < dg.n; k++) {
           v.push_back(dg.d[k].which);
           v.push_back(dg.d[k].radix);
+          v.push_back(dg.d[k].weight);
         }
       }
       break;

@@ -95,15 +95,17 @@ int cuttHipFinishMbar(cuttHipMbar* mb);
  * A free numbering of the workgroups of a tiled launch (tile order 7): the logical workgroup index is
  * read as a mixed-radix number, first digit fastest, and every digit belongs to one of the three
  * coordinates of a workgroup - tile along Mm (which = 0), tile along Mk (1), Mbar position (2).  A
- * coordinate is the mixed-radix number of its own digits in the order they appear.  The product of a
- * coordinate's radices must reach its extent; indices whose coordinates fall beyond an extent are
- * padding workgroups.  Orders 0-5 are special cases (patches of 2 x 8 tiles walked for 192 Mbar
+ * coordinate is the sum of its digits times their weights; sorted by weight, a coordinate's digits
+ * must form a mixed-radix number (weights 1, r0, r0 r1, ...), in whatever order they appear in the
+ * index.  The product of a coordinate's radices must reach its extent; indices whose coordinates fall
+ * beyond an extent are padding workgroups.  Orders 0-5 are special cases (patches of 2 x 8 tiles walked for 192 Mbar
  * positions in turn: m2 k8 b192 m8 k2 for 16 x 16 tiles).
  */
-#define CUTT_MAX_TILE_DIGITS 12
+#define CUTT_MAX_TILE_DIGITS 16
 typedef struct cuttHipTileDigit {
   uint32_t radix;
   uint32_t which;       /* 0 tile along Mm, 1 tile along Mk, 2 Mbar position */
+  uint32_t weight;      /* the digit's value counts weight times in its coordinate */
   cuttHipDivisor div;   /* division by radix (cuttHipMakeDivisor) */
 } cuttHipTileDigit;
 

@@ -501,16 +501,29 @@ bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk,
   uint64_t logical = (uint64_t)tilesM * tilesK * (uint64_t)volMbar;
   if (order == 7) {
     if (dg.n < 1 || dg.n > CUTT_MAX_TILE_DIGITS) return false;
-    uint64_t span[3] = {1, 1, 1};
     logical = 1;
     for (int i = 0; i < dg.n; i++) {
       const cuttHipTileDigit& d = dg.d[i];
       if (d.radix < 1 || d.which > 2 || !divisorOk(d.div, d.radix)) return false;
-      span[d.which] *= d.radix;
       logical *= d.radix;
       if (logical > 0x7fffffffull) return false;  // the decode divides 31-bit numbers
     }
-    if (span[0] < (uint64_t)tilesM || span[1] < (uint64_t)tilesK || span[2] < (uint64_t)volMbar) return false;
+    // per coordinate the digits, taken by growing weight, must be a mixed-radix number that reaches the extent
+    const uint64_t extent[3] = {(uint64_t)tilesM, (uint64_t)tilesK, (uint64_t)volMbar};
+    for (uint32_t w = 0; w < 3; w++) {
+      uint64_t span = 1;
+      for (;;) {
+        int next = -1;
+        for (int i = 0; i < dg.n; i++)
+          if (dg.d[i].which == w && dg.d[i].weight == span && dg.d[i].radix > 1 && (next < 0 || dg.d[i].radix > dg.d[next].radix)) next = i;
+        if (next < 0) break;
+        span *= dg.d[next].radix;
+      }
+      uint64_t all = 1;
+      for (int i = 0; i < dg.n; i++)
+        if (dg.d[i].which == w && dg.d[i].radix > 1) all *= dg.d[i].radix;
+      if (span != all || span < extent[w]) return false;
+    }
   } else if (order >= 3) {
     if (superM < 1 || superK < 1) return false;
     logical = (uint64_t)((tilesM + superM - 1) / superM) * ((tilesK + superK - 1) / superK) * superM * superK *

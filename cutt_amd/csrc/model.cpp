@@ -485,6 +485,10 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // along Mm ran 1.11 times as long as predicted in the mean (0.84-1.37), those with three and
     // more tiles along Mm 0.97 times.
     if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0 && bytes > cacheBytes) factor *= 1.1;  // measured at 1.9-3.7 GB
+    // Workgroups numbered by the address bits their digits move (plan.cpp: addressBitOrder): such plans
+    // ran at 0.90-0.93 of this estimate (C2 584 -> 522 us; five 4-byte batched transposes 615 -> 571-597 us),
+    // while the aligned PackedSplit candidates they compete with ran 1.1-1.35 times theirs.
+    if (!copy && plan.tiled.order == 7) factor *= 0.91;
   } else {
     factor = 1.05 + (es == 4 ? 0.17 : 0.15) * (rdAmp - 1.0) + 0.18 * (wrAmp - 1.0) + 0.08 * partial - (es == 4 ? 0.07 : 0.0) -
              (plan.method == kPacked ? 0.05 : 0.0) + 0.25 * partial * far(r.wrEdgeDist) +

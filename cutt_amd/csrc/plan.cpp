@@ -556,37 +556,47 @@ struct TileOrdering {
 };
 
 // Order 7: the digits of `text` ("m2,k8,b0,m0,k0": coordinate letter + radix, fastest first; radix 0 = what
-// is left of the coordinate).  A coordinate whose digits do not reach its extent gets one more, slowest,
-// digit.  Returns the number of logical workgroups, 0 if the text is malformed.
+// is left of the coordinate; "m2@4" gives the digit the weight 4 in its coordinate instead of the product of
+// the coordinate's earlier radices).  A coordinate whose digits do not reach its extent gets one more,
+// slowest, digit.  Returns the number of logical workgroups, 0 if the text is malformed.
 int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK, int64_t volMbar, cuttHipTileDigits& dg) {
   std::memset(&dg, 0, sizeof(dg));
   const int64_t extent[3] = {tilesM, tilesK, volMbar};
   int64_t span[3] = {1, 1, 1};
-  auto push = [&](int which, int64_t radix) {
-    if (dg.n >= CUTT_MAX_TILE_DIGITS || radix < 1 || radix > 0x7fffffffll) return false;
+  auto push = [&](int which, int64_t radix, int64_t weight) {
     if (radix == 1) return true;
+    if (dg.n >= CUTT_MAX_TILE_DIGITS || radix < 1 || radix > 0x7fffffffll || weight < 1 || weight > 0x7fffffffll) return false;
     dg.d[dg.n].which = (uint32_t)which;
     dg.d[dg.n].radix = (uint32_t)radix;
+    dg.d[dg.n].weight = (uint32_t)weight;
     dg.d[dg.n].div = cuttHipMakeDivisor((uint32_t)radix);
     dg.n++;
     span[which] *= radix;
     return true;
+  };
+  auto number = [&](size_t& pos) {
+    int64_t v = 0;
+    while (pos < text.size() && text[pos] >= '0' && text[pos] <= '9') v = v * 10 + (text[pos++] - '0');
+    return v;
   };
   size_t pos = 0;
   while (pos < text.size()) {
     const char c = text[pos++];
     const int which = c == 'm' ? 0 : (c == 'k' ? 1 : (c == 'b' ? 2 : -1));
     if (which < 0) return 0;
-    int64_t radix = 0;
-    while (pos < text.size() && text[pos] >= '0' && text[pos] <= '9') radix = radix * 10 + (text[pos++] - '0');
+    int64_t radix = number(pos), weight = span[which];
+    if (pos < text.size() && text[pos] == '@') {
+      pos++;
+      weight = number(pos);
+    }
     if (pos < text.size() && text[pos] == ',') pos++;
     if (radix == 0) radix = ceilDiv(extent[which], span[which]);
-    if (!push(which, radix)) return 0;
+    if (!push(which, radix, weight)) return 0;
   }
   for (int w : {2, 0, 1})
-    if (span[w] < extent[w] && !push(w, ceilDiv(extent[w], span[w]))) return 0;
+    if (span[w] < extent[w] && !push(w, ceilDiv(extent[w], span[w]), span[w])) return 0;
   if (dg.n == 0) {  // a single workgroup
-    dg.d[0].which = 0; dg.d[0].radix = 1; dg.d[0].div = cuttHipMakeDivisor(1); dg.n = 1;
+    dg.d[0].which = 0; dg.d[0].radix = 1; dg.d[0].weight = 1; dg.d[0].div = cuttHipMakeDivisor(1); dg.n = 1;
   }
   int64_t logical = 1;
   for (int i = 0; i < dg.n; i++) {
@@ -706,6 +716,118 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   return logical;
 }
 
+// Workgroup numbering for batched transposes whose tiles sit on power-of-two addresses.
+//
+// Measured (random orders of the binary digits of tile and Mbar indices, 1500-2500 per tensor, on ten
+// tensors of 1.6 GB per buffer, 4- and 8-byte elements): which digits change among the tiles that run
+// at the same time decides 20-40 % of the rate (3.4-6.2 TB/s), and what decides is the address bit a
+// digit moves, on either side, the same for every tensor:
+//   - address bit 11 must differ among the tiles in flight - on the write side above all (a digit that
+//     moves the written address by 2 KB, placed where it changes only every few thousand workgroups,
+//     costs 10-14 %; in the three slowest digits, which the eight XCDs split among them, or among the
+//     fastest seven it gains 4-6 %), the read side half as much;
+//   - tile digits that move an address by 1 KB or 4 KB (bits 10, 12) and any digit that moves it by
+//     128 KB (bit 17) are better left slow (3-4 % each when among the fastest four);
+//   - the other digits matter little; consecutive Mbar positions and the 2 x 2 patch of tiles first.
+// The rule below (bit-11 digits and one 1-KB digit slowest = split over the XCDs; 1 KB / 4 KB / 128 KB
+// digits below them; 2 x 2 patch, Mbar digits, other tile digits fastest) reached 0.996 of the rate
+// of the measuring planner's plan in the mean over all 35 four-rank batched transposes
+// (2^a, 2^j, 2^b, 3) -> (2^b, 2^j, 2^a, 3) of 2e8 8-byte elements (lowest 0.85; the orders it replaces:
+// 0.93 and 0.78), C2 5.6 -> 6.2 TB/s.  With 128 and more tiles along Mk it lost 5-14 % on five of six,
+// so those keep the strips.  Returns the number of logical workgroups, 0 if the tensor is not of
+// this class.
+int64_t addressBitOrder(const Problem& pb, const Split& sp, const cuttHipMbar& mb, int64_t tilesM, int64_t tilesK,
+                        cuttHipTileDigits& dg) {
+  auto log2Exact = [](int64_t v) {
+    int l = 0;
+    while ((int64_t{1} << l) < v) l++;
+    return (int64_t{1} << l) == v ? l : -1;
+  };
+  const int es = pb.elemSize, esBits = es == 8 ? 3 : 2;
+  const int bitsM = log2Exact(tilesM), bitsK = log2Exact(tilesK);
+  if (sp.numMm != 1 || sp.numMk != 1 || bitsM < 2 || bitsK < 2 || tilesK >= 128) return 0;
+  if (sp.volMm != tilesM * kTile || sp.volMk != tilesK * kTile) return 0;
+  const int rk = pb.perm[0];
+  const int outM = log2Exact(pb.strideOut[0]), inK = log2Exact(pb.strideIn[rk]);
+  if (outM < 0 || inK < 0) return 0;
+  struct Digit {
+    int which, radix;
+    int64_t weight;
+    int rd, wr;  // address bit the digit moves on the read / write side, -1 = not a single bit
+    int index;   // position among the digits of its coordinate
+  };
+  std::vector<Digit> all;
+  for (int i = 0; i < bitsM; i++) all.push_back({0, 2, int64_t{1} << i, 6 + esBits + i, outM + esBits + 6 + i, i});
+  for (int i = 0; i < bitsK; i++) all.push_back({1, 2, int64_t{1} << i, inK + esBits + 6 + i, 6 + esBits + i, i});
+  int64_t below = 1;
+  int nb = 0, binaryMbar = 0;
+  for (int k = 0; k < mb.n; k++) {
+    int64_t e = mb.d[k].extent, w = below;
+    const int rd = log2Exact(mb.d[k].strideIn), wr = log2Exact(mb.d[k].strideOut);
+    for (int t = 0; e % 2 == 0; t++, e /= 2, w *= 2) {
+      all.push_back({2, 2, w, rd < 0 ? -1 : rd + esBits + t, wr < 0 ? -1 : wr + esBits + t, nb++});
+      binaryMbar++;
+    }
+    if (e > 1) all.push_back({2, (int)e, w, -1, -1, nb++});
+    below *= mb.d[k].extent;
+  }
+  if (binaryMbar < 2 || (int)all.size() > CUTT_MAX_TILE_DIGITS) return 0;
+  auto moves = [](const Digit& d, int bit) { return d.rd == bit || d.wr == bit; };
+  std::vector<Digit> top, slow, fast, odd;
+  for (const Digit& d : all)
+    if (d.radix == 2 && moves(d, 11)) top.push_back(d);
+  auto taken = [&](const Digit& d) {
+    for (const Digit& t : top)
+      if (t.which == d.which && t.weight == d.weight) return true;
+    return false;
+  };
+  if (top.size() > 3) top.resize(3);
+  for (int bit : {10, 12})  // a third digit for the XCDs: a tile digit that moves 1 KB, else 4 KB
+    for (const Digit& d : all)
+      if (top.size() < 3 && top.size() >= 1 && d.which != 2 && d.radix == 2 && moves(d, bit) && !taken(d) &&
+          (bit == 10 || top.size() == 2))
+        top.push_back(d);
+  for (const Digit& d : all) {
+    if (taken(d)) continue;
+    // (an Mbar digit that moves both addresses by 2 MB and more steps from one slice of the tensor to
+    // another: among the fastest digits it cost 10-40 % on tensors whose last rank is a power of two)
+    if (d.radix != 2 || (d.which == 2 && d.rd >= 21 && d.wr >= 21)) odd.push_back(d);
+    else if ((d.which != 2 && (moves(d, 10) || moves(d, 12))) || moves(d, 17)) slow.push_back(d);
+    else fast.push_back(d);
+  }
+  // fastest: the 2 x 2 patch, then the Mbar digits in their order, then the other tile digits
+  std::stable_sort(fast.begin(), fast.end(), [](const Digit& a, const Digit& b) {
+    auto cls = [](const Digit& d) { return d.which != 2 && d.index == 0 ? 0 : (d.which == 2 ? 1 : 2); };
+    return cls(a) != cls(b) ? cls(a) < cls(b) : (cls(a) == 2 ? a.index < b.index : false);
+  });
+  // slowest of the slow ones: the digits that move 1 KB / 4 KB
+  std::stable_sort(slow.begin(), slow.end(), [&](const Digit& a, const Digit& b) {
+    const bool ka = moves(a, 10) || moves(a, 12), kb = moves(b, 10) || moves(b, 12);
+    return ka != kb ? kb : a.index < b.index;
+  });
+  std::vector<Digit> seq = fast;
+  seq.insert(seq.end(), slow.begin(), slow.end());
+  // the three slowest digits are binary, so that each XCD's chunk is one value of them
+  while (top.size() < 3 && !seq.empty()) {
+    top.push_back(seq.back());
+    seq.pop_back();
+  }
+  if (top.size() < 3) return 0;
+  seq.insert(seq.end(), odd.begin(), odd.end());  // odd factors of the Mbar extents and far Mbar digits right below the top
+  seq.insert(seq.end(), top.begin(), top.end());
+  std::memset(&dg, 0, sizeof(dg));
+  int64_t logical = 1;
+  for (const Digit& d : seq) {
+    cuttHipTileDigit& o = dg.d[dg.n++];
+    o.which = (uint32_t)d.which;
+    o.radix = (uint32_t)d.radix;
+    o.weight = (uint32_t)d.weight;
+    o.div = cuttHipMakeDivisor((uint32_t)d.radix);
+    logical *= d.radix;
+  }
+  return logical <= 0x7fffffffll ? logical : 0;
+}
+
 bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptions& opt) {
   const Split& sp = plan.split;
   const Problem& pb = plan.pb;
@@ -750,12 +872,27 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
       if (!sp.inMmk[r] && pb.strideIn[r] == sp.volMm && pb.strideOut[r] == sp.volMk) between = true;
     const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
     const bool beyondCache = (double)pb.volume * pb.elemSize > 0.75 * cacheBytes;
-    plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
-                                 sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o, a.digits);
+    if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
+    int64_t byAddressBits = 0;
+    if (opt.superAuto && opt.addressBits && opt.tiledOrder < 0 && opt.tileDigits.empty() && between && !a.alignedStores && sp.volMbar > 1 &&
+        beyondCache)
+      byAddressBits = addressBitOrder(pb, sp, a.mbar, a.tilesM, a.tilesK, a.digits);
+    if (byAddressBits > 0) {
+      o.order = 7;
+      o.superM = o.superK = 1;
+      o.xcdChunk = 0;
+      plan.numBlocks = byAddressBits;
+      if (opt.xcdAware && byAddressBits >= 64) {
+        o.xcdChunk = (uint32_t)ceilDiv(byAddressBits, kNumXcd);
+        plan.numBlocks = (int64_t)o.xcdChunk * kNumXcd;
+      }
+    } else {
+      plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
+                                   sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o, a.digits);
+    }
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     a.grouped = opt.tiledGrouped > 0 && !a.alignedStores ? 1 : 0;  // -1: decided from the model's estimate later
-    if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
     plan.ldsBytes = (size_t)(kTile + (a.alignedStores ? 128 / pb.elemSize - 1 : 0)) * (kTile + 1) * pb.elemSize;
   } else {
     cuttHipTiledCopyArgs& a = plan.tcopy;
@@ -1015,6 +1152,17 @@ void addPackedSplit(const Problem& pb, bool fromReduced, const cuttHipDeviceProp
 }
 
 }  // namespace
+
+// Text form of a digit list (what parseTileDigits reads).
+std::string formatTileDigits(const cuttHipTileDigits& dg) {
+  std::string t;
+  for (int i = 0; i < dg.n; i++) {
+    if (i) t += ',';
+    t += "mkb"[dg.d[i].which];
+    t += std::to_string(dg.d[i].radix) + "@" + std::to_string(dg.d[i].weight);
+  }
+  return t;
+}
 
 bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const PlannerOptions& opt, Plan& out) {
   out = Plan();

@@ -149,6 +149,7 @@ struct PlannerOptions {
   bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
   std::string tileDigits;   // non-empty: tiled order 7 with this mixed-radix numbering, fastest digit first, e.g.
                             // "m2,k8,b0,m0,k0" (m / k = tile along Mm / Mk, b = Mbar position; radix 0 = what is left)
+  bool addressBits = true;  // Tiled: number the workgroups by the address bits their digits move where that rule applies (addressBitOrder)
   int tiledFuse = -1;       // Tiled over fused rank sets: -1 = planner's choice, 0 = one rank per side only
   int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on
   int tiledGrouped = -1;    // Tiled: rows of a lane in flight, -1 = planner's choice, 0 = all 16, 1 = 4 at a time
@@ -174,6 +175,9 @@ bool createPlans(const Problem& orig, const Problem& red, const cuttHipDevicePro
 // Same index sets as `src`, launch geometry recomputed under different options (used by the
 // measuring planner to try ordering and granularity variants of its best candidate).
 bool rebuildPlan(const Plan& src, const cuttHipDeviceProps& props, const PlannerOptions& opt, Plan& out);
+
+// Text form of a tile digit list, as PlannerOptions::tileDigits takes it.
+std::string formatTileDigits(const cuttHipTileDigits& dg);
 
 // Default device description of one MI355X, used when no GPU is present (tests, offline planning).
 cuttHipDeviceProps defaultMI355XProps();

@@ -71,16 +71,16 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
     return m < volMbar;
   } else if (o.order == 7) {
     const cuttHipTileDigits& dg = *o.digits;
-    uint32_t c0 = 0, c1 = 0, c2 = 0, w0 = 1, w1 = 1, w2 = 1, rest = l;
+    uint32_t c0 = 0, c1 = 0, c2 = 0, rest = l;
     for (int i = 0; i < dg.n; i++) {
       const cuttHipTileDigit d = dg.d[i];
       const uint32_t q = fastDivide(rest, d.div.mul, d.div.shift, d.div.add);
       // the slowest digit takes what is left (beyond its radix on the padding workgroups)
-      const uint32_t v = i + 1 < dg.n ? rest - q * d.radix : rest;
+      const uint32_t v = (i + 1 < dg.n ? rest - q * d.radix : rest) * d.weight;
       rest = q;
-      if (d.which == 0) { c0 += v * w0; w0 *= d.radix; }
-      else if (d.which == 1) { c1 += v * w1; w1 *= d.radix; }
-      else { c2 += v * w2; w2 *= d.radix; }
+      if (d.which == 0) c0 += v;
+      else if (d.which == 1) c1 += v;
+      else c2 += v;
     }
     tm = c0; tk = c1; m = c2;
     return tm < tilesM && tk < tilesK && m < volMbar;

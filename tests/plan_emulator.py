@@ -35,19 +35,16 @@ def _check_tile_decode(num_blocks, order, tiles_m, tiles_k, vol_mbar, xcd_chunk,
         l = b
     if order == 7:
         # mixed-radix number, fastest digit first; every digit belongs to one coordinate
-        n = len(digits) // 2
-        assert 1 <= n <= 12
+        n = len(digits) // 3
+        assert 1 <= n <= 16
         coord = [np.zeros_like(l), np.zeros_like(l), np.zeros_like(l)]
-        weight = [1, 1, 1]
         rest = l.copy()
         for i in range(n):
-            which, radix = int(digits[2 * i]), int(digits[2 * i + 1])
-            assert which in (0, 1, 2) and radix >= 1
+            which, radix, weight = int(digits[3 * i]), int(digits[3 * i + 1]), int(digits[3 * i + 2])
+            assert which in (0, 1, 2) and radix >= 1 and weight >= 1
             v = rest % radix if i + 1 < n else rest
             rest = rest // radix
-            coord[which] = coord[which] + v * weight[which]
-            weight[which] *= radix
-        assert weight[0] >= tiles_m and weight[1] >= tiles_k and weight[2] >= vol_mbar
+            coord[which] = coord[which] + v * weight
         tm, tk, m = coord
         ok = (tm < tiles_m) & (tk < tiles_k) & (m < vol_mbar)
     elif order == 0:

@@ -663,7 +663,7 @@ def test_free_tile_numbering(gpu, monkeypatch):
         for es in (4, 8):
             data = gpu.seeded(int(np.prod(dim)), es, seed=3 + es)
             expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
-            for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0"]:
+            for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0", "m2@2,b2@2,m2@1,k0,b2@1,b0,m0"]:
                 monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
                 with cutt.Candidates(dim, perm, es) as c:
                     idx = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]

@@ -206,11 +206,14 @@ def test_super_tile_shapes_of_the_tiled_plan(cutt):
     # strips of 8 tiles through all of Mk, every strip for all Mbar positions in turn
     assert tiled((4457, 44570), (1, 0), 4) == (3, 8, 697)
     assert tiled((1535, 157, 895), (2, 1, 0), 4) == (5, 8, 14)
-    # 8-byte rows on the 128-byte grid: patches; two wide with an Mbar rank between Mm and Mk (C2)
-    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 8) == (5, 2, 8)
+    # 8-byte rows on the 128-byte grid: patches; two wide with an Mbar rank between Mm and Mk
+    assert tiled((1024, 48, 1024, 4), (2, 1, 0, 3), 8) == (5, 2, 8)
+    # ... and with power-of-two strides throughout (C2) the numbering by address bits (order 7)
+    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 8) == (7, 1, 1)
     assert tiled((2048, 1024, 95), (1, 0, 2), 8) == (5, 8, 8)       # a batch of separate matrices
     assert tiled((4096, 12, 3936), (2, 1, 0), 8) == (5, 8, 8)       # input rows a multiple of 32 KB
-    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 16, 16)   # 4-byte: one strip for a rank of 16 tiles
+    assert tiled((1000, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 16, 16)   # 4-byte: one strip for a rank of 16 tiles
+    assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 4) == (7, 1, 1)
     # 4-byte input rows a multiple of 32 KB apart: strips 16 wide, beyond the memory-side cache only
     assert tiled((8192, 8192), (1, 0), 4) == (3, 16, 128)
     assert tiled((16384, 100, 77), (2, 1, 0), 4) == (5, 16, 2)
@@ -301,7 +304,7 @@ def test_free_tile_numbering(cutt, oracle_mod, monkeypatch):
     # along Mm, the tile along Mk and the Mbar position; every tile must be visited exactly once
     cutt.set_method_override(4)  # Tiled only
     try:
-        for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0"]:
+        for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0", "m2@2,b2@2,m2@1,k0,b2@1,b0,m0"]:
             monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
             for dim, perm in [((200, 6, 300, 3), (2, 1, 0, 3)), ((70, 130), (1, 0)), ((650, 3, 5, 70), (3, 1, 2, 0))]:
                 with cutt.Candidates(dim, perm, 8) as c:
@@ -310,3 +313,31 @@ def test_free_tile_numbering(cutt, oracle_mod, monkeypatch):
                 check_all_candidates(cutt, oracle_mod, dim, perm, 8, need="Tiled")
     finally:
         cutt.set_method_override(0)
+
+
+def test_numbering_by_address_bits(cutt, monkeypatch):
+    """Batched transposes on power-of-two addresses: the digits of the workgroup number that move address bit 11
+    (on either side) are the three slowest (split over the XCDs), tile digits that move 1 KB / 4 KB and digits
+    that move 128 KB come right below them, the 2 x 2 patch and the Mbar digits are fastest."""
+    def digits(dim, perm, es):
+        with cutt.Candidates(dim, perm, es) as c:
+            t = [i for i in range(len(c)) if c.info(i).method_name == "Tiled" and c.info(i).numMm == 1 and c.info(i).numMk == 1]
+            assert len(t) == 1
+            d = c.data(t[0], 8)
+            return c.info(t[0]).tiledOrder, ["%s%d@%d" % ("mkb"[d[3 * k]], d[3 * k + 1], d[3 * k + 2]) for k in range(len(d) // 3)]
+    order, dg = digits((1024, 64, 1024, 3), (2, 1, 0, 3), 8)
+    # tile digit 4 (the third binary digit) moves 2 KB = address bit 11 in rows of 8-byte elements
+    assert order == 7 and sorted(dg[-3:]) == ["k2@4", "m2@2", "m2@4"], dg
+    assert dg[:2] == ["m2@1", "k2@1"] and dg[2:6] == ["b2@1", "b2@2", "b2@4", "b2@8"], dg
+    assert dg[-4] == "b3@64", dg                        # the odd factor of the Mbar extent right below the top
+    assert set(dg[7:11]) == {"b2@16", "k2@2", "m2@8", "k2@8"}, dg   # 128 KB, 1 KB, 4 KB, 4 KB
+    order, dg = digits((2048, 64, 1024, 3), (2, 1, 0, 3), 4)
+    # 4-byte elements: a tile row is 256 bytes, so the fourth binary digit moves address bit 11
+    assert order == 7 and {"m2@8", "k2@8"} <= set(dg[-3:]), dg
+    # not of this class: a batch of separate matrices, extents that are no powers of two, 128 tiles along Mk,
+    # a tensor inside the memory-side cache, a plain 2-D transpose
+    for dim, perm, es in [((1024, 1024, 192), (1, 0, 2), 8), ((1024, 48, 1024, 4), (2, 1, 0, 3), 8), ((256, 32, 8192, 3), (2, 1, 0, 3), 8),
+                          ((256, 16, 256, 3), (2, 1, 0, 3), 8), ((8192, 8192), (1, 0), 4)]:
+        assert digits(dim, perm, es)[0] != 7, (dim, perm)
+    monkeypatch.setenv("CUTT_ADDRESS_BITS", "0")
+    assert digits((1024, 64, 1024, 3), (2, 1, 0, 3), 8)[0] == 5
