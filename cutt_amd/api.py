@@ -114,6 +114,8 @@ def lib():
     l.cuttCountAddressStream.argtypes = [ctypes.c_uint, ctypes.c_int, ctypes.POINTER(StreamCounts),
                                          ctypes.POINTER(StreamCounts)]
     l.cuttCountAddressStream.restype = ctypes.c_int
+    l.cuttDeviceCallCounts.argtypes = [ctypes.POINTER(ctypes.c_ulonglong), ctypes.POINTER(ctypes.c_ulonglong)]
+    l.cuttDeviceCallCounts.restype = None
     l.cuttSetMethodOverride.argtypes = [ctypes.c_int]
     l.cuttSetMethodOverride.restype = None
     l.cuttGetMethodOverride.argtypes = []
@@ -222,6 +224,13 @@ def count_address_stream(handle, num_samples=0):
 
 def set_method_override(method):
     lib().cuttSetMethodOverride(int(method))
+
+
+def device_call_counts():
+    """(device allocations, table uploads) the library has made in this process so far."""
+    a, u = ctypes.c_ulonglong(0), ctypes.c_ulonglong(0)
+    lib().cuttDeviceCallCounts(ctypes.byref(a), ctypes.byref(u))
+    return a.value, u.value
 
 
 def clear_plan_cache():

@@ -672,11 +672,13 @@ static cuttResult measureProblem(const Problem& orig, const Problem& red, int fo
   if (!estimateAll(plans, props)) return CUTT_INTERNAL_ERROR;
   for (Plan& p : plans) chooseCachePolicy(p, props);
 
-  // Candidates the model puts far behind its best are not timed (its error is well inside that
-  // margin); CUTT_MEASURE_ALL=1 times every candidate, as the reference does.
+  // Candidates the model puts more than twice behind its best are not timed when there are many (the
+  // model's worst recorded errors: classes of plans that ran 1.3-1.4 times their estimate, a pick at 0.6 of
+  // the measured plan's rate); up to twenty candidates are all timed, as the reference does with any
+  // number (src/cutt.cpp:236-262), and CUTT_MEASURE_ALL=1 asks for that always.
   double bestPred = 1e300;
   for (const Plan& p : plans) bestPred = std::min(bestPred, p.model.usPredicted);
-  double margin = 1.6;
+  double margin = plans.size() <= 20 ? 1e30 : 2.0;
   if (const char* e = std::getenv("CUTT_MEASURE_ALL"))
     if (std::atoi(e) != 0) margin = 1e30;
 
@@ -1039,22 +1041,30 @@ extern "C" int cuttGetMethodOverride(void) {
 }
 
 extern "C" int cuttGetLastMeasurement(cuttPlanInfo* infos, int maxInfos) {
-  std::lock_guard<std::mutex> lock(gMutex);
-  const int n = (int)gLastMeasurement.size();
-  for (int i = 0; i < n && i < maxInfos && infos; i++) infos[i] = gLastMeasurement[i];
-  return n;
+  try {
+    std::lock_guard<std::mutex> lock(gMutex);
+    const int n = (int)gLastMeasurement.size();
+    for (int i = 0; i < n && i < maxInfos && infos; i++) infos[i] = gLastMeasurement[i];
+    return n;
+  } catch (...) {  // nothing may cross the C boundary
+    return -1;
+  }
 }
 
 extern "C" int cuttReduceRanks(int rank, const int* dim, const int* permutation, int* redDim,
                                int* redPermutation) {
-  if (rank < 1 || !dim || !permutation || !redDim || !redPermutation) return -1;
-  std::vector<int> d, p;
-  reduceRanks(rank, dim, permutation, d, p);
-  for (size_t i = 0; i < d.size(); i++) {
-    redDim[i] = d[i];
-    redPermutation[i] = p[i];
+  try {
+    if (rank < 1 || !dim || !permutation || !redDim || !redPermutation) return -1;
+    std::vector<int> d, p;
+    reduceRanks(rank, dim, permutation, d, p);
+    for (size_t i = 0; i < d.size(); i++) {
+      redDim[i] = d[i];
+      redPermutation[i] = p[i];
+    }
+    return (int)d.size();
+  } catch (...) {  // nothing may cross the C boundary
+    return -1;
   }
-  return (int)d.size();
 }
 
 namespace {
@@ -1064,6 +1074,10 @@ struct CandidateList {
 };
 }  // namespace
 
+extern "C" void cuttDeviceCallCounts(unsigned long long* allocations, unsigned long long* uploads) {
+  cuttHipCallCounts(allocations, uploads);
+}
+
 extern "C" void cuttClearPlanCache(void) {
   std::lock_guard<std::mutex> lock(gMutex);
   gDecisionIndex.clear();
@@ -1072,73 +1086,79 @@ extern "C" void cuttClearPlanCache(void) {
 
 extern "C" void* cuttCandidatesCreateEx(int rank, const int* dim, const int* permutation,
                                         size_t sizeofType, size_t ldsPerBlock) {
-  if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS) return nullptr;
-  int force;
-  {
-    std::lock_guard<std::mutex> lock(gMutex);
-    force = methodOverrideLocked();
-  }
-  CandidateList* l = new CandidateList();
-  cuttHipDeviceProps props = defaultMI355XProps();
-  if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
-  if (!enumerate(rank, dim, permutation, sizeofType, props, force, l->plans)) {
-    delete l;
+  try {
+    if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS) return nullptr;
+    int force;
+    {
+      std::lock_guard<std::mutex> lock(gMutex);
+      force = methodOverrideLocked();
+    }
+    std::unique_ptr<CandidateList> l(new CandidateList());
+    cuttHipDeviceProps props = defaultMI355XProps();
+    if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
+    if (!enumerate(rank, dim, permutation, sizeofType, props, force, l->plans)) return nullptr;
+    if (!estimateAll(l->plans, props)) return nullptr;
+    l->best = chooseHeuristic(l->plans);
+    return l.release();
+  } catch (...) {  // nothing may cross the C boundary
     return nullptr;
   }
-  if (!estimateAll(l->plans, props)) {
-    delete l;
-    return nullptr;
-  }
-  l->best = chooseHeuristic(l->plans);
-  return l;
 }
 
 extern "C" void* cuttCandidatesCreateStrided(int rank, const int* dim, const int* permutation, size_t sizeofType,
                                              const long long* strideIn, const long long* strideOut,
                                              size_t ldsPerBlock) {
-  if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS || !strideIn || !strideOut) return nullptr;
-  int force;
-  {
-    std::lock_guard<std::mutex> lock(gMutex);
-    force = methodOverrideLocked();
+  try {
+    if (checkInput(rank, dim, permutation, sizeofType) != CUTT_SUCCESS || !strideIn || !strideOut) return nullptr;
+    int force;
+    {
+      std::lock_guard<std::mutex> lock(gMutex);
+      force = methodOverrideLocked();
+    }
+    std::vector<int64_t> sIn(strideIn, strideIn + rank), sOut(strideOut, strideOut + rank);
+    Problem pb;
+    if (!pb.setStrided(rank, dim, permutation, (int)sizeofType, sIn.data(), sOut.data())) return nullptr;
+    std::unique_ptr<CandidateList> l(new CandidateList());
+    cuttHipDeviceProps props = defaultMI355XProps();
+    if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
+    if (!createPlans(pb, pb, props, plannerOptions(force), l->plans) || !estimateAll(l->plans, props)) return nullptr;
+    l->best = chooseHeuristic(l->plans);
+    return l.release();
+  } catch (...) {  // nothing may cross the C boundary
+    return nullptr;
   }
-  std::vector<int64_t> sIn(strideIn, strideIn + rank), sOut(strideOut, strideOut + rank);
-  Problem pb;
-  if (!pb.setStrided(rank, dim, permutation, (int)sizeofType, sIn.data(), sOut.data())) return nullptr;
-  std::unique_ptr<CandidateList> l(new CandidateList());
-  cuttHipDeviceProps props = defaultMI355XProps();
-  if (ldsPerBlock) props.ldsPerBlock = props.ldsPerCU = ldsPerBlock;
-  if (!createPlans(pb, pb, props, plannerOptions(force), l->plans) || !estimateAll(l->plans, props)) return nullptr;
-  l->best = chooseHeuristic(l->plans);
-  return l.release();
 }
 
 extern "C" long long cuttSlabDecomposition(int rank, const int* dim, const int* permutation, size_t sizeofType,
                                            long long spanLimit, long long* values, long long maxCount) {
-  bool large = false;
-  if (checkInput(rank, dim, permutation, sizeofType, &large) != CUTT_SUCCESS) return -1;
-  std::vector<int> redDim, redPerm;
-  reduceRanks(rank, dim, permutation, redDim, redPerm);
-  SlabDecomposition dec;
-  if (!slabDecompose((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType,
-                     spanLimit > 0 ? spanLimit : slabSpanLimit(), dec))
+  try {
+    bool large = false;
+    if (checkInput(rank, dim, permutation, sizeofType, &large) != CUTT_SUCCESS) return -1;
+    std::vector<int> redDim, redPerm;
+    reduceRanks(rank, dim, permutation, redDim, redPerm);
+    SlabDecomposition dec;
+    if (!slabDecompose((int)redDim.size(), redDim.data(), redPerm.data(), (int)sizeofType,
+                       spanLimit > 0 ? spanLimit : slabSpanLimit(), dec))
+      return -1;
+    std::vector<long long> v = {(long long)dec.shapes.size(), (long long)dec.pieces.size()};
+    for (const Problem& p : dec.shapes) {
+      v.push_back(p.rank);
+      for (int r = 0; r < p.rank; r++) v.push_back(p.dim[r]);
+      for (int r = 0; r < p.rank; r++) v.push_back(p.perm[r]);
+      for (int r = 0; r < p.rank; r++) v.push_back(p.strideIn[r]);
+      for (int r = 0; r < p.rank; r++) v.push_back(p.strideOut[r]);
+    }
+    for (const SlabPiece& q : dec.pieces) {
+      v.push_back(q.shape);
+      v.push_back(q.baseIn);
+      v.push_back(q.baseOut);
+    }
+    if (values)
+      for (long long i = 0; i < std::min<long long>(maxCount, (long long)v.size()); i++) values[i] = v[i];
+    return (long long)v.size();
+  } catch (...) {  // nothing may cross the C boundary
     return -1;
-  std::vector<long long> v = {(long long)dec.shapes.size(), (long long)dec.pieces.size()};
-  for (const Problem& p : dec.shapes) {
-    v.push_back(p.rank);
-    for (int r = 0; r < p.rank; r++) v.push_back(p.dim[r]);
-    for (int r = 0; r < p.rank; r++) v.push_back(p.perm[r]);
-    for (int r = 0; r < p.rank; r++) v.push_back(p.strideIn[r]);
-    for (int r = 0; r < p.rank; r++) v.push_back(p.strideOut[r]);
   }
-  for (const SlabPiece& q : dec.pieces) {
-    v.push_back(q.shape);
-    v.push_back(q.baseIn);
-    v.push_back(q.baseOut);
-  }
-  if (values)
-    for (long long i = 0; i < std::min<long long>(maxCount, (long long)v.size()); i++) values[i] = v[i];
-  return (long long)v.size();
 }
 
 extern "C" void* cuttCandidatesCreate(int rank, const int* dim, const int* permutation,
@@ -1160,83 +1180,87 @@ extern "C" int cuttCandidatesInfo(void* list, int index, cuttPlanInfo* info) {
 
 extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                                         long long maxCount) {
-  CandidateList* l = (CandidateList*)list;
-  if (!l || index < 0 || index >= (int)l->plans.size() || cls < 0 || cls > 3) return -1;
-  const Plan& p = l->plans[index];
-  std::vector<long long> v;
-  const bool packed = p.method == kPacked || p.method == kPackedSplit;
-  switch (what) {
-    case 0: {
-      const cuttHipMbar& mb = packed ? p.packed.mbar : (p.method == kTiled ? p.tiled.mbar : p.tcopy.mbar);
-      if (p.method == kTrivial) break;
-      for (int k = 0; k < mb.n; k++) {
-        v.push_back(mb.d[k].extent);
-        v.push_back(mb.d[k].strideIn);
-        v.push_back(mb.d[k].strideOut);
-      }
-    } break;
-    case 1:
-      if (p.method == kTiled)
-        v = {p.tiled.volMm, p.tiled.volMk, p.tiled.strideInK, p.tiled.strideOutM, p.tiled.tilesM,
-             p.tiled.tilesK, p.tiled.volMbar, p.tiled.order, p.tiled.xcdChunk, p.tiled.superM, p.tiled.superK};
-      else if (p.method == kTiledCopy)
-        v = {p.tcopy.volMm, p.tcopy.volMk, p.tcopy.strideInK, p.tcopy.strideOutK, p.tcopy.tilesM,
-             p.tcopy.tilesK, p.tcopy.volMbar, p.tcopy.order, p.tcopy.xcdChunk, p.tcopy.superM, p.tcopy.superK};
-      else
+  try {
+    CandidateList* l = (CandidateList*)list;
+    if (!l || index < 0 || index >= (int)l->plans.size() || cls < 0 || cls > 3) return -1;
+    const Plan& p = l->plans[index];
+    std::vector<long long> v;
+    const bool packed = p.method == kPacked || p.method == kPackedSplit;
+    switch (what) {
+      case 0: {
+        const cuttHipMbar& mb = packed ? p.packed.mbar : (p.method == kTiled ? p.tiled.mbar : p.tcopy.mbar);
+        if (p.method == kTrivial) break;
+        for (int k = 0; k < mb.n; k++) {
+          v.push_back(mb.d[k].extent);
+          v.push_back(mb.d[k].strideIn);
+          v.push_back(mb.d[k].strideOut);
+        }
+      } break;
+      case 1:
+        if (p.method == kTiled)
+          v = {p.tiled.volMm, p.tiled.volMk, p.tiled.strideInK, p.tiled.strideOutM, p.tiled.tilesM,
+               p.tiled.tilesK, p.tiled.volMbar, p.tiled.order, p.tiled.xcdChunk, p.tiled.superM, p.tiled.superK};
+        else if (p.method == kTiledCopy)
+          v = {p.tcopy.volMm, p.tcopy.volMk, p.tcopy.strideInK, p.tcopy.strideOutK, p.tcopy.tilesM,
+               p.tcopy.tilesK, p.tcopy.volMbar, p.tcopy.order, p.tcopy.xcdChunk, p.tcopy.superM, p.tcopy.superK};
+        else
+          return -1;
+        break;
+      case 2:
+        if (!packed) return -1;
+        v = {p.packed.numThreads, p.packed.volMbar, p.packed.itemsPerBlock, p.packed.padShift,
+             p.packed.ldsElems, p.packed.xcdChunk, p.packed.elemsPerThread, p.packed.itemOrder};
+        for (int i = 0; i < 2; i++) {
+          const cuttHipSplitRank& sr = p.packed.split[i];
+          v.insert(v.end(), {sr.numSplit, sr.slabFloor, sr.slabRem, sr.strideIn, sr.strideOut});
+        }
+        break;
+      case 3: {
+        if (!packed) return -1;
+        const cuttHipPackedClass& k = p.packed.cls[cls];
+        v = {k.vol, k.inCont, k.outCont};
+      } break;
+      case 4:
+        if (!packed) return -1;
+        v.assign(p.tab[cls].rowIn.begin(), p.tab[cls].rowIn.end());
+        break;
+      case 5:
+        if (!packed) return -1;
+        v.assign(p.tab[cls].rowOut.begin(), p.tab[cls].rowOut.end());
+        break;
+      case 6:
+        if (!packed) return -1;
+        v.assign(p.tab[cls].shIdx.begin(), p.tab[cls].shIdx.end());
+        break;
+      case 7:  // Tiled: (extent, stride) of the ranks a tile axis runs over: cls 0 = Mk (input strides), 1 = Mm (output strides)
+        if (p.method != kTiled || cls > 1) return -1;
+        {
+          const cuttHipRowRadix& rr = cls == 0 ? p.tiled.rowsK : p.tiled.rowsM;
+          for (int k = 0; k < rr.n; k++) {
+            v.push_back(rr.extent[k]);
+            v.push_back(rr.stride[k]);
+          }
+        }
+        break;
+      case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix, weight) of the digits, fastest first
+        if (p.method != kTiled && p.method != kTiledCopy) return -1;
+        {
+          const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
+          for (int k = 0; k < dg.n; k++) {
+            v.push_back(dg.d[k].which);
+            v.push_back(dg.d[k].radix);
+            v.push_back(dg.d[k].weight);
+          }
+        }
+        break;
+      default:
         return -1;
-      break;
-    case 2:
-      if (!packed) return -1;
-      v = {p.packed.numThreads, p.packed.volMbar, p.packed.itemsPerBlock, p.packed.padShift,
-           p.packed.ldsElems, p.packed.xcdChunk, p.packed.elemsPerThread, p.packed.itemOrder};
-      for (int i = 0; i < 2; i++) {
-        const cuttHipSplitRank& sr = p.packed.split[i];
-        v.insert(v.end(), {sr.numSplit, sr.slabFloor, sr.slabRem, sr.strideIn, sr.strideOut});
-      }
-      break;
-    case 3: {
-      if (!packed) return -1;
-      const cuttHipPackedClass& k = p.packed.cls[cls];
-      v = {k.vol, k.inCont, k.outCont};
-    } break;
-    case 4:
-      if (!packed) return -1;
-      v.assign(p.tab[cls].rowIn.begin(), p.tab[cls].rowIn.end());
-      break;
-    case 5:
-      if (!packed) return -1;
-      v.assign(p.tab[cls].rowOut.begin(), p.tab[cls].rowOut.end());
-      break;
-    case 6:
-      if (!packed) return -1;
-      v.assign(p.tab[cls].shIdx.begin(), p.tab[cls].shIdx.end());
-      break;
-    case 7:  // Tiled: (extent, stride) of the ranks a tile axis runs over: cls 0 = Mk (input strides), 1 = Mm (output strides)
-      if (p.method != kTiled || cls > 1) return -1;
-      {
-        const cuttHipRowRadix& rr = cls == 0 ? p.tiled.rowsK : p.tiled.rowsM;
-        for (int k = 0; k < rr.n; k++) {
-          v.push_back(rr.extent[k]);
-          v.push_back(rr.stride[k]);
-        }
-      }
-      break;
-    case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix, weight) of the digits, fastest first
-      if (p.method != kTiled && p.method != kTiledCopy) return -1;
-      {
-        const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
-        for (int k = 0; k < dg.n; k++) {
-          v.push_back(dg.d[k].which);
-          v.push_back(dg.d[k].radix);
-          v.push_back(dg.d[k].weight);
-        }
-      }
-      break;
-    default:
-      return -1;
+    }
+    for (long long i = 0; i < (long long)v.size() && i < maxCount && values; i++) values[i] = v[(size_t)i];
+    return (long long)v.size();
+  } catch (...) {  // nothing may cross the C boundary
+    return -1;
   }
-  for (long long i = 0; i < (long long)v.size() && i < maxCount && values; i++) values[i] = v[(size_t)i];
-  return (long long)v.size();
 }
 
 extern "C" int cuttModelGlTransactionsSeg(const int* seg, int n) { return glTransactions(seg, n); }

@@ -274,6 +274,9 @@ int cuttHipGetDevice(int* device);
 int cuttHipGetDeviceProps(int device, cuttHipDeviceProps* props);
 int cuttHipMalloc(void** ptr, size_t bytes);
 int cuttHipFree(void* ptr);
+/* How often this process has called cuttHipMalloc and cuttHipMemcpyHtoD so far (tests read them
+ * before and after a call that must neither allocate nor upload). */
+void cuttHipCallCounts(unsigned long long* mallocs, unsigned long long* uploads);
 /* Host to device copy that has completed when the call returns. */
 int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes);
 int cuttHipMemcpyDtoDAsync(void* dst, const void* src, size_t bytes, void* stream);

@@ -9,9 +9,12 @@
  */
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cstring>
 
 #include "hip_layer.h"
+
+static std::atomic<unsigned long long> gMallocCalls{0}, gUploadCalls{0};
 
 extern "C" int cuttHipGetDevice(int* device) { return (int)hipGetDevice(device); }
 
@@ -39,10 +42,18 @@ extern "C" int cuttHipGetDeviceProps(int device, cuttHipDeviceProps* p) {
   return 0;
 }
 
-extern "C" int cuttHipMalloc(void** ptr, size_t bytes) { return (int)hipMalloc(ptr, bytes); }
+extern "C" int cuttHipMalloc(void** ptr, size_t bytes) {
+  gMallocCalls++;
+  return (int)hipMalloc(ptr, bytes);
+}
+extern "C" void cuttHipCallCounts(unsigned long long* mallocs, unsigned long long* uploads) {
+  if (mallocs) *mallocs = gMallocCalls;
+  if (uploads) *uploads = gUploadCalls;
+}
 extern "C" int cuttHipFree(void* ptr) { return (int)hipFree(ptr); }
 
 extern "C" int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes) {
+  gUploadCalls++;
   return (int)hipMemcpy(dst, src, bytes, hipMemcpyHostToDevice);
 }
 

@@ -39,19 +39,36 @@ bool slabDecompose(int rank, const int* dim, const int* perm, int elemSize, int6
   // Extent of every rank inside one piece.  Per side, from the slowest rank down: a rank whose
   // faster ranks alone exceed the limit is fixed to one index; the first rank that fits partly is
   // cut to the largest extent that fits, and the span is within the limit.
+  // The rank that leads a side (stride 1 there) is passed over as long as the other ranks can bring
+  // the span down: a piece in which that rank had a single entry left would have no contiguous rows
+  // on that side - (3, 40000, 40000) -> (40000, 40000, 3) cuts ranks 1 and 2 into four equal
+  // pieces, where cutting rank 0 into 2 + 1 left a piece that no kernel can address.
   std::vector<int64_t> e(dim, dim + rank);
-  auto shrink = [&](const std::vector<int64_t>& stride, auto rankAt) {
-    for (int j = rank - 1; j >= 0; j--) {
-      int64_t span = 1;
-      for (int r = 0; r < rank; r++) span += (e[r] - 1) * stride[r];
-      if (span <= spanLimit) return;
-      const int r = rankAt(j);
-      const int64_t rest = span - (e[r] - 1) * stride[r];
-      e[r] = rest > spanLimit ? 1 : std::min<int64_t>(e[r], (spanLimit - rest) / stride[r] + 1);
+  const int leadIn = 0, leadOut = perm[0];
+  auto spanOf = [&](const std::vector<int64_t>& stride) {
+    int64_t span = 1;
+    for (int r = 0; r < rank; r++) span += (e[r] - 1) * stride[r];
+    return span;
+  };
+  // Three attempts per side: without either leading rank; without the other side's leading rank (this
+  // side's own leading rank has stride 1 here, its pieces keep whole rows); with every rank.
+  auto shrink = [&](const std::vector<int64_t>& stride, auto rankAt, int ownLead, int otherLead) {
+    for (int pass = 0; pass < 3; pass++) {
+      const std::vector<int64_t> before = e;
+      for (int j = rank - 1; j >= 0; j--) {
+        const int64_t span = spanOf(stride);
+        if (span <= spanLimit) return;
+        const int r = rankAt(j);
+        if ((pass == 0 && r == ownLead) || (pass <= 1 && r == otherLead)) continue;
+        const int64_t rest = span - (e[r] - 1) * stride[r];
+        e[r] = rest > spanLimit ? 1 : std::min<int64_t>(e[r], (spanLimit - rest) / stride[r] + 1);
+      }
+      if (spanOf(stride) <= spanLimit) return;
+      if (pass < 2) e = before;
     }
   };
-  shrink(sIn, [&](int j) { return j; });
-  shrink(sOut, [&](int j) { return perm[j]; });
+  shrink(sIn, [&](int j) { return j; }, leadIn, leadOut);
+  shrink(sOut, [&](int j) { return perm[j]; }, leadOut, leadIn);
 
   // Pieces per rank, evened out so that the last piece is not a sliver.
   std::vector<int64_t> count(rank), last(rank);
@@ -66,7 +83,7 @@ bool slabDecompose(int rank, const int* dim, const int* perm, int elemSize, int6
     numPieces *= count[r];
     if (numPieces > (1ll << 20)) return false;
   }
-  if (odd.size() > 2) return false;  // cannot happen: one cut rank per side
+  if (odd.size() > 2) return false;  // more shapes of piece than a plan holds
 
   // One shape per combination of "last piece or not" of the ranks in `odd`.
   const int numShapes = 1 << odd.size();

@@ -58,8 +58,10 @@ typedef enum cuttResult_t {
  * Sizes: up to 64 ranks and 2^46 elements.  One kernel launch addresses fewer than 2^32 elements;
  * a larger tensor (the reference's int volumes end at 2^31 - 1) is cut into pieces, and
  * cuttExecute issues one launch per piece on the plan's stream.  CUTT_INVALID_PARAMETER beyond
- * those sizes and for the rare shapes in which the fastest rank of the input lies 2^32 elements
- * and more apart in the output (or the other way round).
+ * those sizes and for the shapes that have no such piece: those in which the rank that is
+ * contiguous in the input lies 2^32 elements and more apart in the output, or the other way round -
+ * (2, 70000, 70000) -> (70000, 70000, 2), 34 ranks of extent 2 reversed - and those in which a rank of
+ * 2^31 entries and more has only tiny ranks beside it ((3, 2^31 - 1) transposed).
  */
 cuttResult cuttPlan(cuttHandle* handle, int rank, int* dim, int* permutation,
                     size_t sizeofType, hipStream_t stream);

@@ -93,6 +93,13 @@ int cuttGetMethodOverride(void);
 void cuttClearPlanCache(void);
 
 /*
+ * How often this process has allocated device memory and uploaded index tables on the library's
+ * behalf so far (every cuttPlan of a Packed / PackedSplit plan does both once).  A caller that must
+ * not allocate reads them around cuttExecuteNoAlloc: they do not move.  No counterpart in the reference.
+ */
+void cuttDeviceCallCounts(unsigned long long* allocations, unsigned long long* uploads);
+
+/*
  * After cuttPlanMeasure: the candidates of its most recent call in this
  * process, in enumeration order (a variant of the winner that beat it is
  * appended at the end).  usMeasured is 0 for candidates that were not timed

@@ -8,7 +8,9 @@
 #include <chrono>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 #include <thread>
+#include <vector>
 
 #include "hip_layer.h"
 
@@ -17,6 +19,10 @@ cuttHipDeviceProps defaultMI355XProps();
 }
 
 static std::atomic<uint64_t> gSink;
+static std::atomic<unsigned long long> gMallocCalls{0}, gUploadCalls{0};
+// The index tables of the most recent packed "launch", class by class: rowIn, rowOut, shIdx.
+static std::vector<uint32_t> gLastTables;
+static std::mutex gLastTablesLock;
 
 static void touch(const cuttHipPackedArgs* a) {
   uint64_t sum = 0;
@@ -28,6 +34,17 @@ static void touch(const cuttHipPackedArgs* a) {
     for (int i = 0; i < k.vol; i++) sum += k.shIdx[i];
   }
   gSink = sum;
+  {
+    std::lock_guard<std::mutex> guard(gLastTablesLock);
+    gLastTables.clear();
+    for (int c = 0; c < 4; c++) {
+      if (((c & 1) && a->split[0].slabRem == 0) || ((c & 2) && a->split[1].slabRem == 0)) continue;
+      const cuttHipPackedClass& k = a->cls[c];
+      gLastTables.insert(gLastTables.end(), k.rowIn, k.rowIn + k.vol / k.inCont);
+      gLastTables.insert(gLastTables.end(), k.rowOut, k.rowOut + k.vol / k.outCont);
+      gLastTables.insert(gLastTables.end(), k.shIdx, k.shIdx + k.vol);
+    }
+  }
   std::this_thread::sleep_for(std::chrono::microseconds(50));
 }
 
@@ -39,9 +56,19 @@ int cuttHipGetDeviceProps(int, cuttHipDeviceProps* p) {
   if (z && std::atoi(z)) p->memClockKHz = p->memBusWidthBits = p->cuCount = p->l2Bytes = p->clockKHz = 0;
   return 0;
 }
-int cuttHipMalloc(void** ptr, size_t bytes) { *ptr = std::malloc(bytes ? bytes : 1); return *ptr ? 0 : 2; }
+int cuttHipMalloc(void** ptr, size_t bytes) { gMallocCalls++; *ptr = std::malloc(bytes ? bytes : 1); return *ptr ? 0 : 2; }
+void cuttHipCallCounts(unsigned long long* mallocs, unsigned long long* uploads) {
+  if (mallocs) *mallocs = gMallocCalls;
+  if (uploads) *uploads = gUploadCalls;
+}
+// (test hook of this stand-in only) copies the tables of the most recent packed launch; returns their length
+size_t fakeLastPackedTables(uint32_t* out, size_t capacity) {
+  std::lock_guard<std::mutex> guard(gLastTablesLock);
+  for (size_t i = 0; i < gLastTables.size() && i < capacity; i++) out[i] = gLastTables[i];
+  return gLastTables.size();
+}
 int cuttHipFree(void* ptr) { std::free(ptr); return 0; }
-int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes) { std::memcpy(dst, src, bytes); return 0; }
+int cuttHipMemcpyHtoD(void* dst, const void* src, size_t bytes) { gUploadCalls++; std::memcpy(dst, src, bytes); return 0; }
 int cuttHipMemcpyDtoDAsync(void* dst, const void* src, size_t bytes, void*) { std::memcpy(dst, src, bytes); return 0; }
 int cuttHipMemsetAsync(void* dst, int value, size_t bytes, void*) { std::memset(dst, value, bytes); return 0; }
 int cuttHipDeviceSynchronize(void) { return 0; }

@@ -3,6 +3,9 @@
 //              on the handle in a loop while the main thread destroys it.  Every call must return
 //              CUTT_SUCCESS or CUTT_INVALID_PLAN, and a sanitizer must stay silent (the plan may be
 //              freed only after the last launch that uses it has been issued).
+//   noalloc  - cuttExecuteNoAlloc with the Packed and the PackedSplit method forced: the layer's counters of
+//              device allocations and table uploads must not move, and the index tables the call builds in the
+//              static scratch memory must equal those cuttPlan uploads for the same tensor.
 //   plans    - prints what cuttPlan chooses for a fixed list of tensors (the test compares the
 //              output for a device that reports its properties with one that reports zeros).
 #include <atomic>
@@ -45,6 +48,51 @@ static int race(int rounds) {
   return bad ? 1 : 0;
 }
 
+extern "C" size_t fakeLastPackedTables(uint32_t* out, size_t capacity);  // fake_hip_layer.cpp
+
+static int noalloc() {
+  struct Case { std::vector<int> dim, perm; int es, method; };
+  const Case cases[] = {
+      {{5, 7, 11, 13, 17}, {4, 2, 0, 1, 3}, 4, CUTT_METHOD_PACKED},   {{12, 9, 31, 40}, {2, 0, 3, 1}, 8, CUTT_METHOD_PACKED},
+      {{20000, 2, 50}, {2, 1, 0}, 8, CUTT_METHOD_PACKEDSPLIT},        {{331, 7, 257, 3}, {2, 1, 0, 3}, 4, CUTT_METHOD_PACKEDSPLIT},
+      {{6, 5, 9, 31}, {2, 0, 3, 1}, 4, CUTT_METHOD_PACKED},           {{300, 7, 290}, {2, 1, 0}, 8, CUTT_METHOD_TILED},
+  };
+  std::vector<char> in(64), out(64);
+  int bad = 0;
+  for (const Case& c : cases) {
+    std::vector<int> d = c.dim, p = c.perm;
+    cuttSetMethodOverride(c.method);
+    unsigned long long m0, u0, m1, u1;
+    cuttDeviceCallCounts(&m0, &u0);
+    if (cuttExecuteNoAlloc((int)d.size(), d.data(), p.data(), (size_t)c.es, 0, in.data(), out.data()) != CUTT_SUCCESS) return 1;
+    cuttDeviceCallCounts(&m1, &u1);
+    if (m1 != m0 || u1 != u0) {
+      std::printf("cuttExecuteNoAlloc allocated %llu times, uploaded %llu times\n", m1 - m0, u1 - u0);
+      bad++;
+    }
+    if (c.method == CUTT_METHOD_TILED) continue;  // no tables
+    std::vector<uint32_t> built(1 << 20), uploaded(1 << 20);
+    const size_t nBuilt = fakeLastPackedTables(built.data(), built.size());
+    cuttHandle h;
+    if (cuttPlan(&h, (int)d.size(), d.data(), p.data(), (size_t)c.es, 0) != CUTT_SUCCESS) return 1;
+    cuttPlanInfo info;
+    if (cuttGetPlanInfo(h, &info) != CUTT_SUCCESS || info.method != c.method) return 1;
+    cuttDeviceCallCounts(&m0, &u0);
+    if (m0 != m1 + 1 || u0 != u1 + 1) bad++;  // cuttPlan does allocate and upload: the counters work
+    if (cuttExecute(h, in.data(), out.data()) != CUTT_SUCCESS) return 1;
+    const size_t nUploaded = fakeLastPackedTables(uploaded.data(), uploaded.size());
+    cuttDestroy(h);
+    if (nBuilt == 0 || nBuilt != nUploaded || std::memcmp(built.data(), uploaded.data(), nBuilt * sizeof(uint32_t)) != 0) {
+      std::printf("tables differ: %zu entries built in place, %zu uploaded\n", nBuilt, nUploaded);
+      bad++;
+    }
+    std::printf("method %d: %zu table entries equal, no allocation\n", c.method, nBuilt);
+  }
+  cuttSetMethodOverride(0);
+  std::printf("noalloc done, failures %d\n", bad);
+  return bad ? 1 : 0;
+}
+
 static int plans() {
   struct Case { std::vector<int> dim, perm; int es; };
   const Case cases[] = {
@@ -71,6 +119,7 @@ static int plans() {
 int main(int argc, char** argv) {
   if (argc > 2 && !std::strcmp(argv[1], "race")) return race(std::atoi(argv[2]));
   if (argc > 1 && !std::strcmp(argv[1], "plans")) return plans();
-  std::printf("usage: plan_lifetime_stress race N | plans\n");
+  if (argc > 1 && !std::strcmp(argv[1], "noalloc")) return noalloc();
+  std::printf("usage: plan_lifetime_stress race N | plans | noalloc\n");
   return 2;
 }

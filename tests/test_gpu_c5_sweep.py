@@ -1,6 +1,7 @@
 """The whole sweep configuration: 50 seeded random tensors of about 2e8 elements, ranks 2-7, 8- and
 4-byte elements alternating, every one planned with cuttPlan and with cuttPlanMeasure, timed with
-the reference's protocol beside a same-size device-to-device copy, every output checked on the
+the reference's protocol beside a same-size device-to-device copy and the library's own copy kernel
+(the ceiling of a streaming kernel, about 1.3 times the runtime's copy), every output checked on the
 device against torch's permute of the index pattern, six of them also against the CPU oracle on
 random bits.  The target - every 8-byte tensor at 70 % of the copy or better - is asserted for both
 planners; plan-creation times are reported."""
@@ -48,10 +49,10 @@ def test_sweep_both_planners_every_tensor():
     worst_heuristic = min(fp64, key=lambda r: r["plan"]["pct"])
     assert worst_measured["measure"]["pct"] >= 70.0, worst_measured
     assert worst_heuristic["plan"]["pct"] >= 70.0, worst_heuristic
-    # the measuring planner must not end up behind the heuristic one by more than timing noise (the same plan
-    # timed twice in one process differs by up to 9 % here: the first launch after an idle gap runs faster)
+    # the measuring planner must not end up behind the heuristic one by more than timing noise (the two plans are
+    # timed in turn, the best of four runs each)
     for r in results:
-        assert r["measure"]["ms"] <= 1.12 * r["plan"]["ms"], r
+        assert r["measure"]["ms"] <= 1.05 * r["plan"]["ms"], r
 
 
 @pytest.mark.parametrize("index", [0, 9, 18, 27, 36, 45])

@@ -80,3 +80,14 @@ def test_zeroed_device_properties_do_not_change_the_plan(tmp_path):
         assert r.returncode == 0, r.stdout[-3000:]
         outs.append(r.stdout)
     assert outs[0] == outs[1] and outs[0].count("method") == 8
+
+
+def test_execute_no_alloc_allocates_nothing_and_builds_the_same_tables(tmp_path):
+    # on the stand-in layer, which counts allocations and uploads and keeps the tables of the last launch
+    exe = str(tmp_path / "plan_lifetime_stress")
+    build_on_fake_layer(exe, ["-fsanitize=address,undefined", "-fno-omit-frame-pointer"])
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0", CUTT_PLAN_CACHE="0")
+    r = subprocess.run([exe, "noalloc"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env, timeout=300)
+    assert r.returncode == 0, r.stdout[-3000:]
+    assert "noalloc done, failures 0" in r.stdout and r.stdout.count("table entries equal") == 5, r.stdout[-3000:]
+    assert "ERROR: AddressSanitizer" not in r.stdout and "runtime error:" not in r.stdout, r.stdout[-3000:]

@@ -94,7 +94,44 @@ def test_ranks_beyond_32(cutt):
     assert len({p[1] for p in pieces}) == len(pieces) and len({p[2] for p in pieces}) == len(pieces)
 
 
+def _check_cover(shapes, pieces, total, limit=2 ** 32):
+    seen = 0
+    for shape, base_in, base_out in pieces:
+        s = shapes[shape]
+        assert s["stride_in"][0] == 1 and 1 in s["stride_out"], s      # contiguous rows on both sides
+        span_in = 1 + sum((d - 1) * st for d, st in zip(s["dim"], s["stride_in"]))
+        span_out = 1 + sum((d - 1) * st for d, st in zip(s["dim"], s["stride_out"]))
+        assert span_in < limit and span_out < limit
+        assert base_in + span_in <= total and base_out + span_out <= total
+        seen += int(np.prod(s["dim"], dtype=np.int64))
+    assert seen == total
+
+
+def test_a_short_leading_rank_that_moves_to_the_back(cutt):
+    """Arrays of structures turned into structures of arrays: the short leading rank of the input is the
+    slowest of the output.  Cutting that rank into 2 + 1 would leave a piece without contiguous input
+    rows; it stays whole and the two long ranks are cut instead."""
+    shapes, pieces = cutt.slab_decomposition([3, 40000, 40000], [2, 1, 0], 4, 0)
+    assert len(pieces) == 4 and len(shapes) == 1 and shapes[0]["dim"] == [3, 20000, 20000]
+    _check_cover(shapes, pieces, 3 * 40000 * 40000)
+    # the same with the short rank leading the output, and with a limit that small tensors reach
+    shapes, pieces = cutt.slab_decomposition([40000, 40000, 3], [2, 1, 0], 8, 0)
+    _check_cover(shapes, pieces, 3 * 40000 * 40000)
+    # (the limit leaves room for all entries of the short rank, which lie far apart on the other side)
+    for dim, perm, limit in [([3, 40, 50], [2, 1, 0], 4500), ([40, 50, 3], [2, 0, 1], 4500), ([5, 4, 60, 70], [3, 2, 1, 0], 70000),
+                             ([2, 90, 80], [1, 2, 0], 8000)]:
+        got = cutt.slab_decomposition(dim, perm, 4, limit)
+        assert got is not None, (dim, perm)
+        assert len(got[1]) > 1
+        _check_cover(got[0], got[1], int(np.prod(dim)), limit=limit + 1)
+
+
 def test_shapes_that_cannot_be_cut_are_refused(cutt):
+    # the fastest rank of the input (2 entries) lies 4.9e9 elements apart in the output: no piece within
+    # 32-bit offsets holds two neighbouring input elements
+    assert cutt.slab_decomposition([2, 70000, 70000], [1, 2, 0], 4, 0) is None
+    # ... and the same seen from the output
+    assert cutt.slab_decomposition([70000, 70000, 2], [2, 0, 1], 4, 0) is None
     # a rank of 2^31 - 1 entries beside one of 3: the piece that fits 32-bit offsets on both sides would
     # have to fix the short rank, and the long one then has stride 3 on one side
     assert cutt.slab_decomposition([3, 2 ** 31 - 1], [1, 0], 4, 0) is None

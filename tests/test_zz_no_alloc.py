@@ -1,6 +1,8 @@
-"""cuttExecuteNoAlloc - plan and execute without allocating on the device - against cuttPlan +
-cuttExecute: same bytes, on calls in a row that reuse the library's static scratch memory (the
-second with a smaller tensor and smaller tables), for every method, and its refusals."""
+"""cuttExecuteNoAlloc - plan and execute without allocating on the device - against the CPU oracle and
+against cuttPlan + cuttExecute: same bytes, on calls in a row that reuse the library's static scratch
+memory (the second with a smaller tensor and smaller tables), for every method; that the call neither
+allocates device memory nor uploads tables (the layer's call counters and the device's free memory do
+not move); and its refusals."""
 import sys
 
 import numpy as np
@@ -41,9 +43,15 @@ def both_ways(gpu, dim, perm, es, seed):
     assert cutt.cuttDestroy(h) == cutt.CUTT_SUCCESS
     out = torch.full_like(d_in, -1)
     say("cuttExecuteNoAlloc dim=%s perm=%s es=%d method %s lds %d" % (dim, perm, es, info.method_name, info.ldsBytes))
+    torch.cuda.synchronize()
+    calls = cutt.device_call_counts()
+    free = torch.cuda.mem_get_info()[0]
     rc = cutt.cuttExecuteNoAlloc(len(dim), dim, perm, es, st, d_in.data_ptr(), out.data_ptr())
     assert rc == cutt.CUTT_SUCCESS, rc
     torch.cuda.synchronize()
+    # nothing allocated, nothing uploaded: the library's own counters and the driver's free memory agree
+    assert cutt.device_call_counts() == calls, (calls, cutt.device_call_counts())
+    assert torch.cuda.mem_get_info()[0] == free
     return data, ref, out, info
 
 
@@ -67,6 +75,7 @@ def test_two_calls_in_a_row_second_smaller(gpu):
 @pytest.mark.parametrize("method", ["tiled", "tiledcopy", "packed", "packedsplit", "trivial"])
 def test_every_method(gpu, method):
     import torch
+    import oracle
     import cutt_amd as cutt
     force = {"tiled": cutt.METHOD_TILED, "tiledcopy": cutt.METHOD_TILEDCOPY, "packed": cutt.METHOD_PACKED,
              "packedsplit": cutt.METHOD_PACKEDSPLIT, "trivial": 0}[method]
@@ -80,6 +89,7 @@ def test_every_method(gpu, method):
     finally:
         cutt.set_method_override(0)
     assert info.method_name.lower() == method
+    assert np.array_equal(gpu.to_host(out, es), oracle.transpose_mt(list(dim), list(perm), data, 8))
     assert torch.equal(out, ref)
     # a second, smaller call with the same method
     small = tuple(max(2, d // 2) for d in dim)
@@ -88,7 +98,23 @@ def test_every_method(gpu, method):
         data, ref, out, info = both_ways(gpu, list(small), list(perm), es, seed=4)
     finally:
         cutt.set_method_override(0)
+    assert np.array_equal(gpu.to_host(out, es), oracle.transpose_mt(list(small), list(perm), data, 8))
     assert torch.equal(out, ref)
+
+
+def test_the_counters_do_see_an_allocating_plan(gpu):
+    # what the checks above rest on: cuttPlan of a plan with index tables allocates once and uploads once
+    import cutt_amd as cutt
+    cutt.set_method_override(cutt.METHOD_PACKED)
+    try:
+        before = cutt.device_call_counts()
+        rc, h = cutt.cuttPlan(4, [12, 9, 31, 40], [2, 0, 3, 1], 8, gpu.stream_handle())
+        assert rc == cutt.CUTT_SUCCESS
+        after = cutt.device_call_counts()
+        cutt.cuttDestroy(h)
+    finally:
+        cutt.set_method_override(0)
+    assert after == (before[0] + 1, before[1] + 1)
 
 
 def test_refusals(gpu, monkeypatch):
