@@ -11,6 +11,6 @@ from .api import (  # noqa: F401
     METHOD_NAMES, METHOD_TRIVIAL, METHOD_PACKED, METHOD_PACKEDSPLIT, METHOD_TILED, METHOD_TILEDCOPY,
     CuttError, PlanInfo, StreamCounts, lib, lib_path,
     cuttPlan, cuttPlanMeasure, cuttPlanFromCandidate, cuttExecute, cuttExecuteNoAlloc, cuttDestroy,
-    get_plan_info, count_address_stream, set_method_override, clear_plan_cache, get_last_measurement, reduce_ranks, Candidates, slab_decomposition,
+    get_plan_info, count_address_stream, set_method_override, clear_plan_cache, device_call_counts, get_last_measurement, reduce_ranks, Candidates, slab_decomposition,
 )
 from .build import build  # noqa: F401

@@ -4,8 +4,10 @@
  * and 32-byte sectors each of them touches, partly written lines, LDS bank-conflict degrees.
  *
  * They take the same arguments and the same grid as the kernel they mirror and derive every
- * address with the same device code (tile order, Mbar decode, division constants, the plan's index
- * tables), but issue no load or store of tensor data; the counts of all wavefronts are added up
+ * address with the device functions that kernel itself calls (tile_order.h: tile order, tile geometry and
+ * row addresses; packed_items.h: work-item orders, item offsets, run tables; mbar_decode.h), but issue
+ * no load or store of tensor data (the instance of the Tiled kernel with line-aligned stores has no
+ * counting kernel: cuttHipCountTiled refuses it); the counts of all wavefronts are added up
  * with atomics.  A test compares them with the host model's walk over the same plan.  Counterpart
  * of the reference's model-validation kernels (src/cuttGpuModelKernel.cu:246-646, countTiled,
  * countPacked, countPackedSplit, countTiledCopy, and the driver :686-782), redone for 64-lane
@@ -29,6 +31,7 @@
 
 #include "hip_layer.h"
 #include "mbar_decode.h"
+#include "packed_items.h"
 #include "tile_order.h"
 
 using namespace cutt;
@@ -164,49 +167,30 @@ __global__ __launch_bounds__(kTileThreads) void countTiledCopyKernel(const cuttH
   flush(c, total);
 }
 
-// Mirrors packedKernel: the same tables, the same work-item numbering, E elements per lane.
+// Mirrors packedKernel: the work items a workgroup takes and where they lie (all three work-item
+// orders), and the lanes' offsets inside a staged block, come from the functions that kernel uses
+// (packed_items.h: packedItems, packedLocate, packedInElem, packedOutElem); E elements per lane.
 __global__ __launch_bounds__(1024) void countPackedKernel(const cuttHipPackedArgs a, unsigned long long* total) {
   const uint32_t tid = threadIdx.x, nt = blockDim.x, lane = tid & 63;
   const uint32_t es = (uint32_t)a.elemSize, words = es / 4;
   const uint32_t E = (uint32_t)a.elemsPerThread;
-  const uint32_t ns0 = a.split[0].numSplit, ns1 = a.split[1].numSplit;
-  const uint32_t ipb = (uint32_t)a.itemsPerBlock;
-  const bool byMbar = a.itemOrder == 1;
-  const uint32_t totalItems = byMbar ? (((uint32_t)a.volMbar + ipb - 1) / ipb) * ns0 * ns1 * ipb : (uint32_t)a.volMbar * ns0 * ns1;
-  uint32_t lb = blockIdx.x;
-  if (a.xcdChunk) lb = (blockIdx.x % kNumXcd) * (uint32_t)a.xcdChunk + blockIdx.x / kNumXcd;
-  const uint32_t w0 = lb * ipb;
-  const uint32_t w1 = min(w0 + ipb, totalItems);
-  const uint32_t rem0 = a.split[0].slabRem, rem1 = a.split[1].slabRem;
+  const PackedItems items = packedItems(a);
   const MbarLane mbarLane = loadMbarLane(a.mbar, lane);
-  const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
   LaneCounts c = {};
-  for (uint32_t w = w0; w < w1; w++) {
-    const uint32_t slab = byMbar ? lb : w;
-    const uint32_t t = fastDivide(slab, div0.mul, div0.shift, div0.add);
-    const uint32_t s0 = slab - t * ns0;
-    uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
-    const uint32_t s1 = t - m * ns1;
-    if (byMbar) m = m * ipb + (w - w0);
-    if (m >= (uint32_t)a.volMbar) break;
-    const int cls = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
-    const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
-    const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
+  for (uint32_t w = 0; w < items.count; w++) {
+    int cls;
     uint32_t offIn, offOut;
-    mbarOffsets(mbarLane, m, offIn, offOut);
-    offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
-    offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
+    packedLocate(a, items, mbarLane, w, cls, offIn, offOut);
     const cuttHipPackedClass& k = a.cls[cls];
     const uint32_t last = (uint32_t)k.vol - 1;
     for (uint32_t j = 0; j < E; j++) {
       const uint32_t pRaw = tid + j * nt, p = min(pRaw, last);
       const bool idle = pRaw - lane > last;  // the wavefront's first lane is already beyond the block
-      const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
-      countAccess(c, false, idle, (uint64_t)offIn + k.rowIn[ri] + (p - ri * (uint32_t)k.inCont), es);
+      countAccess(c, false, idle, (uint64_t)offIn + packedInElem(k, p), es);
+      const uint32_t out = packedOutElem(k, p);
       const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
       const uint32_t col = p - ro * (uint32_t)k.outCont;
-      const uint64_t run = (uint64_t)offOut + k.rowOut[ro];
-      countAccess(c, true, idle, run + col, es);
+      countAccess(c, true, idle, (uint64_t)offOut + out, es);
       if (!idle) {
         // lanes beyond the block repeat the last element's slot: they add to no bank of their own
         const uint32_t bank = ((uint32_t)k.shIdx[p] * words) & 63;
@@ -215,7 +199,7 @@ __global__ __launch_bounds__(1024) void countPackedKernel(const cuttHipPackedArg
         c.maxDegree = max(c.maxDegree, degree);
       }
       // every lane that holds the first element of an output run accounts for the run's two ends
-      uint32_t ends = (pRaw <= last && col == 0) ? partialEnds(run, (uint32_t)k.outCont, es) : 0u;
+      uint32_t ends = (pRaw <= last && col == 0) ? partialEnds((uint64_t)offOut + out, (uint32_t)k.outCont, es) : 0u;
       for (int off = 32; off >= 1; off >>= 1) ends += __shfl_xor(ends, off);
       c.v[kWrPartial] += ends;
     }

@@ -40,6 +40,7 @@
 
 #include "hip_layer.h"
 #include "mbar_decode.h"
+#include "packed_items.h"
 #include "tile_order.h"
 
 using namespace cutt;
@@ -317,31 +318,9 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
 
   const uint32_t tid = threadIdx.x;
   const uint32_t nt = blockDim.x;
-  const uint32_t ns0 = a.split[0].numSplit, ns1 = a.split[1].numSplit;
-  const uint32_t ipb = (uint32_t)a.itemsPerBlock;
-  const bool byMbar = a.itemOrder == 1;  // the workgroup keeps its slabs and walks Mbar positions
-  const uint32_t totalItems = byMbar ? (((uint32_t)a.volMbar + ipb - 1) / ipb) * ns0 * ns1 * ipb
-                                     : (uint32_t)a.volMbar * ns0 * ns1;
-  // XCD-aware numbering: XCD x (= blockIdx.x % 8) walks its own contiguous chunk of the work
-  // items, so that neighbouring slabs and Mbar positions share an L2.
-  uint32_t lb = blockIdx.x;
-  if (a.xcdChunk) lb = (blockIdx.x % kNumXcd) * (uint32_t)a.xcdChunk + blockIdx.x / kNumXcd;
-  // The workgroup's items are the numbers wBase + i * wStride, i < count.  Orders 0 and 1: ipb
-  // consecutive numbers.  Order 2: the workgroups of one XCD take the numbers of their chunk in
-  // turn, so that the items in flight at one time are neighbours and a workgroup's next item lies
-  // a whole round ahead.
-  uint32_t wBase = lb * ipb, wStride = 1;
-  uint32_t count = wBase < totalItems ? min(ipb, totalItems - wBase) : 0;
-  if (a.itemOrder == 2) {
-    const uint32_t chunkBlocks = a.xcdChunk ? (uint32_t)a.xcdChunk : gridDim.x;
-    const uint32_t x = lb / chunkBlocks;
-    const uint32_t chunkStart = x * chunkBlocks * ipb;
-    const uint32_t chunkEnd = min(chunkStart + chunkBlocks * ipb, totalItems);
-    wBase = chunkStart + (lb - x * chunkBlocks);
-    wStride = chunkBlocks;
-    count = wBase < chunkEnd ? (chunkEnd - wBase + wStride - 1) / wStride : 0;
-  }
-  const uint32_t rem0 = a.split[0].slabRem, rem1 = a.split[1].slabRem;
+  // which work items this workgroup handles, and where an item lies: packed_items.h
+  const PackedItems items = packedItems(a);
+  const uint32_t count = items.count;
   const int padShift = a.padShift;
 
   // Lanes whose element index lies beyond the block repeat the block's last element (same
@@ -351,22 +330,9 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   uint32_t shSlot[E];            // byte offset of the LDS slot an output element is taken from
   uint32_t last = 0;             // last element index of the class whose data is being loaded
   const MbarLane mbarLane = loadMbarLane(a.mbar, tid & 63);
-  const cuttHipDivisor div0 = a.split[0].div, div1 = a.split[1].div;
 
-  // The workgroup's i-th item -> slab class and the item's base offsets (all wave-uniform).
   auto locate = [&](uint32_t i, int& c, uint32_t& offIn, uint32_t& offOut) __attribute__((always_inline)) {
-    const uint32_t slab = byMbar ? lb : wBase + i * wStride;
-    const uint32_t t = fastDivide(slab, div0.mul, div0.shift, div0.add);
-    const uint32_t s0 = slab - t * ns0;
-    uint32_t m = fastDivide(t, div1.mul, div1.shift, div1.add);
-    const uint32_t s1 = t - m * ns1;
-    if (byMbar) m = m * ipb + i;
-    c = (s0 < rem0 ? 1 : 0) + (s1 < rem1 ? 2 : 0);
-    const uint32_t p0 = s0 * (uint32_t)a.split[0].slabFloor + min(s0, rem0);
-    const uint32_t p1 = s1 * (uint32_t)a.split[1].slabFloor + min(s1, rem1);
-    mbarOffsets(mbarLane, m, offIn, offOut);
-    offIn += p0 * a.split[0].strideIn + p1 * a.split[1].strideIn;
-    offOut += p0 * a.split[0].strideOut + p1 * a.split[1].strideOut;
+    packedLocate(a, items, mbarLane, i, c, offIn, offOut);
   };
   // The lane's table entries of class c: the read side (input offsets, element count) and the
   // write side (output offsets, LDS gather slots) are fetched separately, because the next item's
@@ -374,30 +340,18 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   auto loadReadSide = [&](int c) __attribute__((always_inline)) {
     const cuttHipPackedClass& k = a.cls[c];
     last = (uint32_t)k.vol - 1;
-    const uint32_t inCont = (uint32_t)k.inCont;
-    const uint32_t* gIn = k.rowIn;
 #pragma unroll
-    for (int j = 0; j < E; j++) {
-      const uint32_t p = min(tid + j * nt, last);
-      const uint32_t ri = fastDivide(p, k.inDiv.mul, k.inDiv.shift, k.inDiv.add);
-      // uniform base + 32-bit lane offset here too (the tables are far smaller than 4 GB)
-      const uint32_t rowI = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gIn) + ri * 4u);
-      inOff[j] = (rowI + (p - ri * inCont)) * kScale;
-    }
+    for (int j = 0; j < E; j++) inOff[j] = packedInElem(k, min(tid + j * nt, last)) * kScale;
   };
   auto loadWriteSide = [&](int c) __attribute__((always_inline)) {
     const cuttHipPackedClass& k = a.cls[c];
     const uint32_t lastP = (uint32_t)k.vol - 1;
-    const uint32_t outCont = (uint32_t)k.outCont;
-    const uint32_t* gOut = k.rowOut;
     const uint16_t* gSh = k.shIdx;
 #pragma unroll
     for (int j = 0; j < E; j++) {
       const uint32_t p = min(tid + j * nt, lastP);
-      const uint32_t ro = fastDivide(p, k.outDiv.mul, k.outDiv.shift, k.outDiv.add);
-      const uint32_t rowO = *reinterpret_cast<const uint32_t*>(reinterpret_cast<const unsigned char*>(gOut) + ro * 4u);
       const uint32_t sh = *reinterpret_cast<const uint16_t*>(reinterpret_cast<const unsigned char*>(gSh) + p * 2u);
-      outOff[j] = (rowO + (p - ro * outCont)) * kScale;
+      outOff[j] = packedOutElem(k, p) * kScale;
       shSlot[j] = sh * (uint32_t)sizeof(T);
     }
   };
@@ -441,12 +395,6 @@ __global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, 
   // gather and the stores of item w, so they overlap, and the wait for them (the memory counter
   // counts loads and stores in issue order) does not also wait for those stores to complete.
   if (count == 0) return;
-  if (byMbar) {
-    // the numbers of this workgroup whose Mbar position lies beyond the rank's end are empty
-    const uint32_t mFirst = fastDivide(fastDivide(lb, div0.mul, div0.shift, div0.add), div1.mul, div1.shift, div1.add) * ipb;
-    if (mFirst >= (uint32_t)a.volMbar) return;
-    count = min(count, (uint32_t)a.volMbar - mFirst);
-  }
   uint32_t w = 0, offIn, offOut;  // index of the item among the workgroup's own
   int cls;
   locate(w, cls, offIn, offOut);

@@ -95,3 +95,28 @@ def test_refusals():
     cutt.cuttDestroy(h)
     with pytest.raises(cutt.CuttError):
         cutt.count_address_stream(123456, 0)
+
+
+def test_counts_agree_for_every_work_item_order(monkeypatch):
+    """The packed kernel's three ways of handing out work items (neighbouring slabs, own slabs over Mbar
+    positions, every B-th item of the XCD's chunk): the counting kernel takes its items from the function the
+    transpose kernel uses, so the totals must equal the host model's for each of them."""
+    import torch
+    import cutt_amd as cutt
+    cutt.lib()
+    st = torch.cuda.current_stream().cuda_stream
+    for dim, perm, es in [((331, 7, 257, 3), (2, 1, 0, 3), 4), ((20000, 2, 50), (2, 1, 0), 8), ((5, 7, 11, 13, 17), (4, 2, 0, 1, 3), 4)]:
+        for order in (0, 1, 2):
+            monkeypatch.setenv("CUTT_ITEM_ORDER", str(order))
+            monkeypatch.setenv("CUTT_MAX_ITEMS", "4")
+            for method in (cutt.METHOD_PACKED, cutt.METHOD_PACKEDSPLIT):
+                cutt.set_method_override(method)
+                try:
+                    rc, h = cutt.cuttPlan(len(dim), list(dim), list(perm), es, st)
+                finally:
+                    cutt.set_method_override(0)
+                if rc != cutt.CUTT_SUCCESS:
+                    continue
+                say("dim=%s perm=%s es=%d item order %d method %d" % (dim, perm, es, order, method))
+                check(cutt, h, "item order %d" % order, 0, es)
+                cutt.cuttDestroy(h)
