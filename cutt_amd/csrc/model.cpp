@@ -412,6 +412,26 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
       r.wrEdgeDist = tilesM > 1 ? 1.0 : (pb.rank > 1 ? mbarDist(pb.perm[1], false) : 0.0);
     } else {
       r.wrEdgeDist = tilesK > 1 ? std::min(superM, tilesM) : (nextOut < pb.rank ? mbarDist(pb.perm[nextOut], false) : 0.0);
+      // The rank that follows the Mk set in the output may be one of the Mm set (a fused Mm axis): the run
+      // next in memory is then the same row of Mk for an Mm index that is `apart` entries on, in another
+      // tile along Mm - in the same strip if that is fewer than superM tiles away, else whole strips later
+      // (a strip is superM x tilesK tiles, in order 5 for every Mbar position).  Measured on seven 8-byte
+      // tensors of the reference's suites whose fused-Mm candidate has one or two tiles along Mk: 1.3-1.55
+      // times the estimate that took this distance for zero.
+      if (plan.split.numMm > 1 && nextOut < pb.rank && pb.perm[nextOut] > 0 && pb.perm[nextOut] < plan.split.numMm) {
+        double apart = 1.0;
+        for (int q = 0; q < pb.perm[nextOut]; q++) apart *= pb.dim[q];
+        const double tilesApart = apart / kTile;
+        double d = 0.0;
+        if (tilesApart >= 1.0)
+          d = tilesApart < superM ? tilesApart : tilesApart * tilesK * (order >= 5 ? (double)plan.split.volMbar : 1.0);
+        if (tilesK > 1) {
+          r.wrEdgeOuter = d;
+          r.wrOuterShare = 1.0 / tilesK;
+        } else {
+          r.wrEdgeDist = d;
+        }
+      }
     }
   }
 
@@ -470,7 +490,8 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
     const double wasteCost = es == 4 && bytes > cacheBytes ? 0.12 : 0.25;
     factor = (es == 4 ? 1.00 : 0.95) + wasteCost * waste + (es == 4 ? 0.2 : 0.4) * (rdAmp - 1.0) +
-             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? (es == 4 ? 0.20 : 0.10) : 0.0) + 0.7 * partial * far(r.wrEdgeDist);
+             (es == 4 ? 0.1 : 0.2) * (wrAmp - 1.0) + (copy ? (es == 4 ? 0.20 : 0.10) : 0.0) +
+             0.7 * partial * ((1.0 - r.wrOuterShare) * far(r.wrEdgeDist) + r.wrOuterShare * far(r.wrEdgeOuter));
     // Tiny slabs of 4-byte elements: with one or two tiles along Mm and exactly two along Mk (a
     // 65..128-long output run cut into a 256-byte piece and a remainder), 46 such plans among 3000
     // random tensors ran 1.29-1.37 times (median) as long as predicted; every other class of tile
@@ -485,6 +506,11 @@ bool estimatePlan(Plan& plan, const cuttHipDeviceProps& props, int numSamples) {
     // along Mm ran 1.11 times as long as predicted in the mean (0.84-1.37), those with three and
     // more tiles along Mm 0.97 times.
     if (!copy && es == 8 && tilesK == 2.0 && tilesM <= 2.0 && bytes > cacheBytes) factor *= 1.1;  // measured at 1.9-3.7 GB
+    // A fused Mm axis with one or two tiles along Mk (output runs of at most 1 KB scattered over the rows of
+    // several ranks): eleven such 8-byte candidates of the reference's suites ran 0.96-1.35 times this
+    // estimate, 1.13 in the mean, and the three that ran 1.2-1.35 times were each picked ahead of a
+    // PackedSplit candidate that was 15-25 % faster.
+    if (!copy && es == 8 && tilesK <= 2.0 && plan.split.numMm > 1 && bytes > cacheBytes) factor *= 1.15;
     // Workgroups numbered by the address bits their digits move (plan.cpp: addressBitOrder): such plans
     // ran at 0.90-0.93 of this estimate (C2 584 -> 522 us; five 4-byte batched transposes 615 -> 571-597 us),
     // while the aligned PackedSplit candidates they compete with ran 1.1-1.35 times theirs.

@@ -608,7 +608,7 @@ int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK,
 
 int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
                     int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, bool mbarBetween,
-                    bool beyondCache, TileOrdering& o, cuttHipTileDigits& dg) {
+                    bool beyondCache, bool neighbourRunsInMm, TileOrdering& o, cuttHipTileDigits& dg) {
   std::memset(&dg, 0, sizeof(dg));
   if (!opt.tileDigits.empty()) {
     const int64_t logical = parseTileDigits(opt.tileDigits, tilesM, tilesK, volMbar, dg);
@@ -632,6 +632,12 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   // after the other, (192,270,27,110)/(3,2,0,1) fp64 went from 3.5 to 4.8 TB/s, C4's Tiled plan from
   // 5.05 to 5.4 TB/s, and nothing measured got slower.
   o.order = opt.tiledOrder >= 0 ? opt.tiledOrder : (volMbar > 1 ? 5 : 3);
+  // ... unless the Mm axis runs over fused ranks of which one follows Mk in the output: the runs that are
+  // neighbours in the output then belong to other rows of the Mm axis, not to the next Mbar position, and
+  // all strips along Mm should pass before the Mbar position moves on (order 3).  Six 8-byte tensors of the
+  // reference's suites whose fused-Mm plan has one or two tiles along Mk: 1015-1257 us in order 5,
+  // 772-862 us in order 3 (554 against 802, 561 against 769 us on two more); a seventh lost 9 %.
+  if (opt.tiledOrder < 0 && neighbourRunsInMm) o.order = 3;
   // One measured exception (forced-Tiled sweep over random shapes, all orders timed): with two
   // tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along Mk should run
   // fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows are written as
@@ -888,7 +894,8 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
       }
     } else {
       plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
-                                   sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache, o, a.digits);
+                                   sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache,
+                                   sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm, o, a.digits);
     }
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
@@ -909,7 +916,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     PlannerOptions copt = opt;
     copt.superAuto = false;  // (the measured exceptions are for the Tiled kernel only)
-    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, o, a.digits);
+    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, false, o, a.digits);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;

@@ -96,6 +96,10 @@ struct ModelResult {
   // Work items between the two workgroups that touch the two sides of a run's end (the next run
   // in memory): small = the shared line is still in the L2 when its other part is accessed.
   double rdEdgeDist = 0, wrEdgeDist = 0;
+  // Tiled over fused rank sets: the output runs of a tile row end where the Mk set ends, and the run that
+  // follows in memory may belong to another row of the Mm axis, many tiles away: its distance, and the share
+  // of the partly written lines that lie at such run ends (the others lie between two tiles along Mk).
+  double wrEdgeOuter = 0, wrOuterShare = 0;
   double usPredicted = 0;              // predicted time in microseconds (ranking key)
 };
 

@@ -57,12 +57,78 @@ def test_heuristic_plans_are_close_to_measured_plans():
              r["measure"]["method"], r["measure"]["gbs"], q))
     ratios = np.array(ratios)
     say("heuristic / measured throughput: median %.3f mean %.3f min %.3f" % (np.median(ratios), ratios.mean(), ratios.min()))
-    # this build: median 0.943-0.945, mean 0.935-0.94; the minimum moves with the machine (0.85 on one MI355X,
-    # 0.78 on another, both from 4-byte PackedSplit plans whose two best candidates the model rates equal), so one
-    # outlier is allowed for and the rest is held to the tighter bound.  (The measured plan also profits from
-    # timing noise in its favour.)
+    # this build: median 0.99, mean 0.977, lowest 0.875 (tiles over fused rank sets and their pricing brought the
+    # mean up from 0.935-0.94; the minimum used to move with the machine, 0.78-0.85, both from 4-byte plans whose
+    # two best candidates the model rates equal), so one outlier is allowed for and the rest is held to the
+    # tighter bound.  (The measured plan also profits from timing noise in its favour.)
     ordered = np.sort(ratios)
-    assert np.median(ratios) >= 0.92
-    assert ratios.mean() >= 0.915
-    assert ordered[1] >= 0.80
-    assert ordered[0] >= 0.70
+    assert np.median(ratios) >= 0.95
+    assert ratios.mean() >= 0.945
+    assert ordered[1] >= 0.85
+    assert ordered[0] >= 0.78
+
+
+def aligned_set(seed=77):
+    """Twelve seeded tensors of about 2e8 elements whose rows start on 128-byte lines on both sides, the class in
+    which the cost model's line counts are the same for nearly all candidates and what decides is which
+    addresses are in flight at one time: four batched transposes (2^a, 2^j, 2^b, 3) -> (2^b, 2^j, 2^a, 3), four
+    tensors of ranks 3-6 whose extents are powers of two (one of them times three), four whose extents are
+    multiples of 32; 8- and 4-byte elements alternating."""
+    rng = np.random.default_rng(seed)
+    out = []
+    while len(out) < 4:
+        a, b = int(rng.integers(8, 13)), int(rng.integers(8, 13))
+        j = 26 - a - b
+        if j < 1:
+            continue
+        out.append(dict(dim=(2 ** a, 2 ** j, 2 ** b, 3), perm=(2, 1, 0, 3)))
+    while len(out) < 8:
+        rank = 3 + len(out) % 4
+        cuts = np.sort(rng.choice(np.arange(1, 26), size=rank - 1, replace=False))
+        bits = np.diff(np.concatenate(([0], cuts, [26])))
+        dim = [int(2 ** e) for e in bits]
+        dim[int(rng.integers(rank))] *= 3
+        perm = [int(p) for p in rng.permutation(rank)]
+        if perm == list(range(rank)) or perm[0] == 0:
+            continue
+        out.append(dict(dim=tuple(dim), perm=tuple(perm)))
+    while len(out) < 12:
+        rank = 3 + len(out) % 3
+        dim = bc.random_dims(rng, rank, target=2.0e8 / 32 ** 2, tol=0.05)
+        perm = [int(p) for p in rng.permutation(rank)]
+        if perm == list(range(rank)) or perm[0] == 0:
+            continue
+        dim = list(dim)
+        dim[0] *= 32            # the rank that leads the input
+        dim[perm[0]] *= 32      # the rank that leads the output
+        out.append(dict(dim=tuple(int(d) for d in dim), perm=tuple(perm)))
+    for i, c in enumerate(out):
+        c["name"] = "A%02d" % i
+        c["es"] = 8 if i % 2 == 0 else 4
+    return out
+
+
+def test_heuristic_plans_on_line_aligned_tensors():
+    """The second set: tensors on the line grid (powers of two above all), where cuttPlan used to reach 0.90 of
+    the measured plan's rate in the mean and 0.61 at worst."""
+    import torch
+    assert torch.cuda.is_available(), "this test needs the MI355X"
+    import cutt_amd
+    import sweep_runner
+    cutt_amd.lib()
+    cutt_amd.set_method_override(0)
+    ratios = []
+    for cfg in aligned_set():
+        r = sweep_runner.run_tensor(cfg, reps=5)
+        assert r["plan"]["exact"] and r["measure"]["exact"], cfg
+        q = r["measure"]["ms"] / r["plan"]["ms"]
+        ratios.append(q)
+        say("%s dim=%s perm=%s es=%d: heuristic %s %.0f GB/s, measured %s %.0f GB/s, ratio %.3f" %
+            (cfg["name"], cfg["dim"], cfg["perm"], cfg["es"], r["plan"]["method"], r["plan"]["gbs"],
+             r["measure"]["method"], r["measure"]["gbs"], q))
+    ratios = np.array(ratios)
+    say("line-aligned set, heuristic / measured throughput: median %.3f mean %.3f min %.3f" %
+        (np.median(ratios), ratios.mean(), ratios.min()))
+    # this build: median 0.961, mean 0.951, lowest 0.868
+    assert ratios.mean() >= 0.925
+    assert ratios.min() >= 0.80
