@@ -310,8 +310,13 @@ __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTil
 // WIDE = false: the tensor is smaller than 4 GB, so the lanes keep 32-bit byte offsets and every
 // access is "uniform 64-bit base + 32-bit lane offset" (no per-access 64-bit address registers).  WIDE = true:
 // element offsets and 64-bit address arithmetic.
+// (The 8-byte instance with 8 elements per lane sits at the edge of a register granule: it is held to the 80
+// registers that let six of its waves share a SIMD; the other instances get what the compiler gives them.)
+template <typename T, int E, bool WIDE>
+constexpr int kPackedMinWaves = (sizeof(T) == 8 && E == 8 && !WIDE) ? 6 : 1;
+
 template <typename T, int E, int NT, bool WIDE>
-__global__ __launch_bounds__(1024) void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
+__global__ __launch_bounds__(1024, (kPackedMinWaves<T, E, WIDE>)) void packedKernel(const cuttHipPackedArgs a, const T* __restrict__ in,
                              T* __restrict__ out) {
   extern __shared__ __align__(16) unsigned char ldsRaw[];
   constexpr uint32_t kScale = WIDE ? 1u : (uint32_t)sizeof(T);

@@ -78,8 +78,8 @@ extern "C" size_t cuttHipPackedLdsBytes(const cuttHipPackedArgs* a) {
 // Registers per lane of packedKernel<T, E, *, WIDE> as compiled for gfx950 (the cache policy does
 // not change the count).  Rows: E = 1, 2, 4, 8, 16.
 extern "C" int cuttHipPackedRegsPerLane(int elemSize, int elemsPerThread, int wideOffsets) {
-  static const int narrow4[5] = {15, 23, 39, 68, 124}, wide4[5] = {18, 25, 40, 72, 128};
-  static const int narrow8[5] = {16, 25, 42, 80, 0}, wide8[5] = {18, 28, 48, 88, 0};
+  static const int narrow4[5] = {15, 23, 38, 68, 124}, wide4[5] = {17, 27, 40, 72, 128};
+  static const int narrow8[5] = {15, 25, 43, 73, 0}, wide8[5] = {18, 28, 48, 88, 0};
   int row = 0;
   while (row < 5 && (1 << row) != elemsPerThread) row++;
   if (row == 5 || (elemSize != 4 && elemSize != 8)) return 0;
