@@ -32,17 +32,19 @@ HBM_PEAK_GBS = 8000.0
 # in runs of their own, each scaled by what the counter reads for the same-size device-to-device
 # copy).  A figure belongs to one launched kernel instance: it is reported only when the plan of
 # this run has the signature (method, workgroups, tile order, super-tile shape, cache policy, rows
-# in groups) the profile was taken on, together with the name of the profile; otherwise null.
+# in groups, digits of the workgroup number in tile order 7) the profile was taken on, together with
+# the name of the profile; otherwise null.
+C2_ADDRESS_BIT_DIGITS = "m2@1,k2@1,b2@1,b2@2,b2@4,b2@8,b2@32,b2@16,k2@2,m2@8,k2@8,b3@64,m2@4,k2@4,m2@2"
 C2_TRAFFIC_PROFILES = {
-    ("Tiled", 49152, 7, 1, 1, 3, 0): (3221375181, "profiles/tiledKernel_u64_C2_address_bit_order.txt"),
-    ("Tiled", 49152, 5, 2, 8, 3, 0): (3221443482, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
-    ("Tiled", 49152, 6, 2, 2, 3, 0): (3221508198, "profiles/tiledKernel_u64_C2_order6_measured_plan.txt"),
+    ("Tiled", 49152, 7, 1, 1, 3, 0, C2_ADDRESS_BIT_DIGITS): (3221375181, "profiles/tiledKernel_u64_C2_address_bit_order.txt"),
+    ("Tiled", 49152, 5, 2, 8, 3, 0, ""): (3221443482, "profiles/tiledKernel_u64_C2_hbm_traffic_pmc.txt"),
+    ("Tiled", 49152, 6, 2, 2, 3, 0, ""): (3221508198, "profiles/tiledKernel_u64_C2_order6_measured_plan.txt"),
 }
 
 
 def plan_signature(info):
     return (info.method_name, int(info.numBlocks), int(info.tiledOrder), int(info.superM), int(info.superK),
-            int(info.cachePolicy), int(info.tiledGrouped))
+            int(info.cachePolicy), int(info.tiledGrouped), info.tileDigits.decode())
 
 
 def log(*a):
@@ -314,6 +316,7 @@ def main():
         "config": {"workload": "C2: fp64 dims (1024,64,1024,3) perm (2,1,0,3), 201326592 elements, value = linear index",
                    "planner": "cuttPlan", "method": info.method_name, "blocks": info.numBlocks,
                    "threads": info.numThreads, "tile_order": info.tiledOrder, "super_tile": [info.superM, info.superK],
+                   "tile_digits": info.tileDigits.decode(),
                    "cache_policy": info.cachePolicy, "plan_ms": round(plan_ms, 2)},
         "pct_of_d2d_memcpy": round(100.0 * value / memcpy_gbs_loop, 1),
         "d2d_memcpy_GBs": round(memcpy_gbs_loop, 1),

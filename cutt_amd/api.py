@@ -54,6 +54,7 @@ class PlanInfo(ctypes.Structure):
         ("tiledGrouped", ctypes.c_int), ("superM", ctypes.c_int), ("superK", ctypes.c_int),
         ("tiledAligned", ctypes.c_int), ("itemOrder", ctypes.c_int),
         ("numPieces", ctypes.c_int), ("numShapes", ctypes.c_int), ("wideOffsets", ctypes.c_int),
+        ("tileDigits", ctypes.c_char * 192),
     ]
 
     @property
@@ -62,6 +63,7 @@ class PlanInfo(ctypes.Structure):
 
     def as_dict(self):
         d = {name: getattr(self, name) for name, _ in self._fields_}
+        d["tileDigits"] = self.tileDigits.decode()
         d["method_name"] = self.method_name
         return d
 

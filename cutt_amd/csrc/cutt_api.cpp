@@ -224,6 +224,11 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   o.superK = p.method == kTiled ? (int)p.tiled.superK : (p.method == kTiledCopy ? (int)p.tcopy.superK : 0);
   o.rdEdgeDist = p.model.rdEdgeDist;
   o.wrEdgeDist = p.model.wrEdgeDist;
+  std::memset(o.tileDigits, 0, sizeof(o.tileDigits));
+  if ((p.method == kTiled || p.method == kTiledCopy) && o.tiledOrder == 7) {
+    const std::string t = formatTileDigits(p.method == kTiled ? p.tiled.digits : p.tcopy.digits);
+    std::strncpy(o.tileDigits, t.c_str(), sizeof(o.tileDigits) - 1);
+  }
 }
 
 void setCachePolicy(Plan& p, int policy) {

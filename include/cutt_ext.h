@@ -38,7 +38,7 @@ typedef struct cuttPlanInfo {
   long long numBlocks;
   int numThreads;
   int itemsPerBlock;    /* Packed/PackedSplit */
-  int tiledOrder;       /* Tiled/TiledCopy: numbering of the workgroups, 0-6 (hip_layer.h: cuttHipTiledArgs.order) */
+  int tiledOrder;       /* Tiled/TiledCopy: numbering of the workgroups, 0-7 (hip_layer.h: cuttHipTiledArgs.order) */
   unsigned long long ldsBytes;
   /* cost model */
   double usPredicted;
@@ -65,6 +65,9 @@ typedef struct cuttPlanInfo {
   int numShapes;        /* different shapes among those pieces (each has a plan of its own): 1..4 */
   int wideOffsets;      /* Packed/PackedSplit: 1 if the kernel instance does 64-bit address arithmetic (the
                            tensor, or the piece of a larger one, spans 4 GB and more) */
+  char tileDigits[192]; /* Tiled/TiledCopy in order 7: the digits of the workgroup number, fastest first, in the
+                           syntax of CUTT_TILE_DIGITS ("m2@1,k2@1,b3@64,..." = coordinate, radix, weight);
+                           empty for the other orders */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */

@@ -107,3 +107,65 @@ def test_sweep_sample_all_methods_agree(gpu):
             assert torch.equal(r, results[0])
         import oracle
         assert np.array_equal(gpu.to_host(results[0], es), oracle.transpose_mt(dim, perm, data, 16))
+
+
+def test_bench_line_reports_traffic_for_the_plan_it_launches(gpu):
+    """bench.py prints the HBM traffic of the C2 kernel only when the plan it launches has a signature one of the
+    committed counter profiles was taken on; the heuristic plan of C2 must be one of them (a change to the planner
+    that alters that plan shows here, and the profile has to be taken again), and the profile must exist."""
+    import os
+    import bench
+    import cutt_amd as cutt
+    cfg = bc.C2
+    rc, h = cutt.cuttPlan(len(cfg["dim"]), list(cfg["dim"]), list(cfg["perm"]), cfg["es"], gpu.stream_handle())
+    assert rc == cutt.CUTT_SUCCESS
+    sig = bench.plan_signature(cutt.get_plan_info(h))
+    cutt.cuttDestroy(h)
+    say("C2 plan signature %s" % (sig,))
+    assert sig in bench.C2_TRAFFIC_PROFILES, sig
+    traffic, source = bench.C2_TRAFFIC_PROFILES[sig]
+    assert os.path.isfile(os.path.join(bench.ROOT, source)), source
+    algorithmic = 2 * cfg["es"] * int(np.prod(cfg["dim"], dtype=np.int64))
+    assert algorithmic <= traffic <= 1.01 * algorithmic
+
+
+def test_default_measuring_planner_against_timing_every_candidate(gpu, monkeypatch):
+    """cuttPlanMeasure skips candidates its model puts far behind when there are more than twenty; the plan it ends
+    with must not be slower than the one found with every candidate timed (CUTT_MEASURE_ALL=1) by more than timing
+    noise.  Three sweep tensors of rank 6-7, whose candidate lists are the long ones."""
+    import torch
+    import cutt_amd as cutt
+    import sweep_runner
+    picked = [c for c in bc.sweep() if len(c["dim"]) >= 6][:3]
+    assert len(picked) == 3
+    for cfg in picked:
+        dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
+        vol = int(np.prod(dim, dtype=np.int64))
+        d_in = sweep_runner.index_pattern(vol, es)
+        d_out = torch.empty_like(d_in)
+        want = sweep_runner.expected_on_device(d_in, dim, perm)
+        st = gpu.stream_handle()
+        handles = {}
+        for name, env in (("default", None), ("all", "1")):
+            if env is None:
+                monkeypatch.delenv("CUTT_MEASURE_ALL", raising=False)
+            else:
+                monkeypatch.setenv("CUTT_MEASURE_ALL", env)
+            say("%s dim=%s perm=%s es=%d: cuttPlanMeasure (%s)" % (cfg["name"], dim, perm, es, name))
+            rc, h = cutt.cuttPlanMeasure(len(dim), dim, perm, es, st, d_in.data_ptr(), d_out.data_ptr())
+            assert rc == cutt.CUTT_SUCCESS
+            timed = sum(1 for i in cutt.get_last_measurement() if i.usMeasured > 0)
+            handles[name] = (h, timed, cutt.get_plan_info(h))
+        monkeypatch.delenv("CUTT_MEASURE_ALL", raising=False)
+        best = {k: float("inf") for k in handles}
+        for _ in range(4):
+            for k, (h, _, _) in handles.items():
+                def execute():
+                    assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+                best[k] = min(best[k], sweep_runner.timed_ms(execute, d_out, 1)[0])
+                assert torch.equal(d_out, want)
+        for k, (h, timed, info) in handles.items():
+            say("  %-7s %s, %d of %d candidates timed, %.3f ms" % (k, info.method_name, timed, info.numCandidates, best[k]))
+            cutt.cuttDestroy(h)
+        assert handles["default"][1] <= handles["all"][1]
+        assert best["default"] <= 1.05 * best["all"], (cfg, best)
