@@ -86,7 +86,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_ITEM_DIGITS", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
@@ -227,6 +227,9 @@ void fillInfo(const Plan& p, cuttPlanInfo& o) {
   std::memset(o.tileDigits, 0, sizeof(o.tileDigits));
   if ((p.method == kTiled || p.method == kTiledCopy) && o.tiledOrder == 7) {
     const std::string t = formatTileDigits(p.method == kTiled ? p.tiled.digits : p.tcopy.digits);
+    std::strncpy(o.tileDigits, t.c_str(), sizeof(o.tileDigits) - 1);
+  } else if ((p.method == kPacked || p.method == kPackedSplit) && p.itemDigits.n > 0) {
+    const std::string t = formatTileDigits(p.itemDigits);
     std::strncpy(o.tileDigits, t.c_str(), sizeof(o.tileDigits) - 1);
   }
 }
@@ -421,6 +424,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_TILED_GROUPED")) opt.tiledGrouped = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILED_ALIGNED")) opt.tiledAligned = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILE_DIGITS")) opt.tileDigits = e;
+  if (const char* e = std::getenv("CUTT_ITEM_DIGITS")) opt.itemDigits = e;
   if (const char* e = std::getenv("CUTT_TILED_FUSE")) opt.tiledFuse = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_ADDRESS_BITS")) opt.addressBits = std::atoi(e) != 0;
   return opt;
@@ -1247,10 +1251,10 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
           }
         }
         break;
-      case 8:  // Tiled / TiledCopy, tile order 7: (coordinate, radix, weight) of the digits, fastest first
-        if (p.method != kTiled && p.method != kTiledCopy) return -1;
+      case 8:  // tile order 7 / work-item order 3: (coordinate, radix, weight) of the digits, fastest first
+        if (p.method != kTiled && p.method != kTiledCopy && !packed) return -1;
         {
-          const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
+          const cuttHipTileDigits& dg = packed ? p.itemDigits : (p.method == kTiled ? p.tiled.digits : p.tcopy.digits);
           for (int k = 0; k < dg.n; k++) {
             v.push_back(dg.d[k].which);
             v.push_back(dg.d[k].radix);

@@ -219,6 +219,7 @@ Plan::Plan() {
   std::memset(&tiled, 0, sizeof(tiled));
   std::memset(&tcopy, 0, sizeof(tcopy));
   std::memset(&packed, 0, sizeof(packed));
+  std::memset(&itemDigits, 0, sizeof(itemDigits));
 }
 
 Plan::~Plan() { release(); }
@@ -237,6 +238,7 @@ Plan& Plan::operator=(Plan&& o) noexcept {
   tiled = o.tiled;
   tcopy = o.tcopy;
   packed = o.packed;
+  itemDigits = o.itemDigits;
   ldsBytes = o.ldsBytes;
   numBlocks = o.numBlocks;
   numThreads = o.numThreads;
@@ -261,6 +263,7 @@ Plan Plan::clone() const {
   q.tiled = tiled;
   q.tcopy = tcopy;
   q.packed = packed;
+  q.itemDigits = itemDigits;
   for (int c = 0; c < 4; c++) {  // device tables stay with the original
     q.packed.cls[c].rowIn = nullptr;
     q.packed.cls[c].rowOut = nullptr;
@@ -317,6 +320,8 @@ void enumerateOffsets(const std::vector<RadixDim>& dims, int64_t count, std::vec
 // remaining index space: mbarOrder 0 = input order (consecutive workgroups read neighbouring
 // memory), 1 = output order (they write neighbouring memory, so the partly written 128-byte
 // lines at the ends of their runs meet in the same L2).
+int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK, int64_t volMbar, cuttHipTileDigits& dg);
+
 bool fillMbar(const Problem& pb, const std::vector<char>& inMmk, int mbarOrder, cuttHipMbar& mb) {
   std::memset(&mb, 0, sizeof(mb));
   // Order of the Mbar ranks (first = fastest over consecutive work items):
@@ -434,6 +439,155 @@ bool shortUnalignedInputRuns(const Split& sp, const Problem& pb, const cuttHipPa
   return false;
 }
 
+// Number the work items of a packed plan by a list of digits (fastest first; which 0 / 1 = slab of the first /
+// second cut rank, 2 = Mbar position; each digit advances its coordinate by its weight).  Needs no kernel
+// support: a work item's offsets are linear in every digit as long as all slabs of a cut rank have one size,
+// so the digits become the entries of the table that the kernel decodes an item number with (the Mbar table:
+// extent = radix, strides = what one step of the digit adds to the two offsets), the cut ranks' slab counts
+// become 1 and the table's positions the work items.  False (and nothing changed) if a cut rank has slabs of
+// two sizes, if the digits of a coordinate are no mixed-radix number of exactly its extent, or if an Mbar digit
+// straddles two ranks.
+bool numberItemsByDigits(cuttHipPackedArgs& a, const cuttHipTileDigits& dg) {
+  if (a.split[0].slabRem || a.split[1].slabRem || dg.n < 1) return false;
+  const int64_t extent[3] = {a.split[0].numSplit, a.split[1].numSplit, a.volMbar};
+  for (uint32_t w = 0; w < 3; w++) {  // per coordinate: weights 1, r1, r1*r2, ... up to the extent
+    int64_t span = 1;
+    for (;;) {
+      int next = -1;
+      for (int i = 0; i < dg.n; i++)
+        if (dg.d[i].which == w && dg.d[i].radix > 1 && (int64_t)dg.d[i].weight == span) next = next < 0 ? i : -2;
+      if (next == -1) break;
+      if (next < 0) return false;  // two digits of one weight
+      span *= dg.d[next].radix;
+    }
+    int64_t all = 1;
+    for (int i = 0; i < dg.n; i++)
+      if (dg.d[i].which == w && dg.d[i].radix > 1) all *= dg.d[i].radix;
+    if (span != all || span != extent[w]) return false;
+  }
+  cuttHipMbar mb;
+  std::memset(&mb, 0, sizeof(mb));
+  int64_t items = 1;
+  for (int i = 0; i < dg.n; i++) {
+    const cuttHipTileDigit& d = dg.d[i];
+    if (d.radix <= 1) continue;
+    if (mb.n >= CUTT_MAX_RANK) return false;
+    int64_t stepIn = 0, stepOut = 0;
+    if (d.which < 2) {
+      const cuttHipSplitRank& sr = a.split[d.which];
+      stepIn = (int64_t)d.weight * sr.slabFloor * (int64_t)sr.strideIn;
+      stepOut = (int64_t)d.weight * sr.slabFloor * (int64_t)sr.strideOut;
+    } else {
+      int64_t below = 1;
+      int k = 0;
+      for (; k < a.mbar.n; below *= a.mbar.d[k].extent, k++)
+        if ((int64_t)d.weight >= below && (int64_t)d.weight < below * a.mbar.d[k].extent) break;
+      if (k == a.mbar.n || (int64_t)d.weight % below != 0) return false;
+      const int64_t u = (int64_t)d.weight / below;
+      if ((int64_t)a.mbar.d[k].extent % (u * d.radix) != 0) return false;  // the digit stays inside rank k
+      stepIn = u * (int64_t)a.mbar.d[k].strideIn;
+      stepOut = u * (int64_t)a.mbar.d[k].strideOut;
+    }
+    if (stepIn > 0xffffffffll || stepOut > 0xffffffffll) return false;
+    mb.d[mb.n].extent = d.radix;
+    mb.d[mb.n].strideIn = (uint32_t)stepIn;
+    mb.d[mb.n].strideOut = (uint32_t)stepOut;
+    mb.n++;
+    items *= d.radix;
+  }
+  if (mb.n < 1 || items > 0x7fffffffll || cuttHipFinishMbar(&mb) != 0) return false;
+  a.mbar = mb;
+  a.volMbar = (int)items;
+  for (int i = 0; i < 2; i++) {
+    a.split[i].numSplit = 1;
+    a.split[i].strideIn = a.split[i].strideOut = 0;
+    a.split[i].div = cuttHipMakeDivisor(1);
+  }
+  a.itemOrder = 0;
+  return true;
+}
+
+// Address bit 11 among the work items that run together.
+//
+// Measured (150 random orders of the binary digits of slab and Mbar indices on each of 30 packed
+// candidates of eight tensors with power-of-two extents, 1.3e8-2.7e8 elements of both widths; rates from
+// 2.8 to 5.9 TB/s on one candidate): one thing stands out of the noise on every candidate, the same that
+// the tiled kernel shows (addressBitOrder).  The digit that moves the read or the written address by 2 KB
+// must not sit where it is constant for everything in flight: at the positions between the digits that
+// the resident workgroups of an XCD differ in and the three slowest digits, which the eight XCDs split
+// among them - all XCDs walk their chunks at the same pace, so such a digit has one value on the whole
+// chip for thousands of work items - it costs 10-20 % (write side) or 5-15 % (read side); any other place
+// is fine, no other digit shows more than the +-5 % of the timing noise.  So: the default numbering (slabs
+// of the first cut rank, of the second, Mbar ranks), with the digits at bit 11 that would lie in that zone
+// moved to the very top.  `residentPerXcd` = workgroups one XCD holds at a time.  False if there is nothing
+// to move (or the numbering cannot be written as at most 16 digits).
+bool thawAddressBit11(const cuttHipPackedArgs& a, int elemSize, int64_t residentPerXcd, cuttHipTileDigits& dg) {
+  if (a.split[0].slabRem || a.split[1].slabRem) return false;
+  auto log2Exact = [](int64_t v) {
+    int l = 0;
+    while ((int64_t{1} << l) < v) l++;
+    return (int64_t{1} << l) == v ? l : -1;
+  };
+  const int esBits = elemSize == 8 ? 3 : 2;
+  struct Part {
+    uint32_t which;
+    int64_t radix, weight;
+    bool bit11;
+  };
+  std::vector<Part> seq;
+  // one entry of the default numbering: a coordinate's rank of `extent` positions, `weight` apart in the
+  // coordinate, whose step moves the two addresses by stepIn / stepOut elements; cut at its bit-11 digit(s)
+  auto add = [&](uint32_t which, int64_t extent, int64_t weight, int64_t stepIn, int64_t stepOut) {
+    if (extent <= 1) return;
+    int cut[2] = {-1, -1};
+    int n = 0;
+    for (int64_t step : {stepIn, stepOut}) {
+      const int l = step > 0 ? log2Exact(step) : -1;
+      const int t = l < 0 ? -1 : 11 - esBits - l;  // the binary digit of this rank that moves byte-address bit 11
+      if (t >= 0 && extent % (int64_t{1} << (t + 1)) == 0 && t != cut[0]) cut[n++] = t;
+    }
+    if (n == 2 && cut[0] > cut[1]) std::swap(cut[0], cut[1]);
+    int64_t done = 1;  // positions of the rank covered so far
+    for (int i = 0; i < n; i++) {
+      const int64_t lowRadix = (int64_t{1} << cut[i]) / done;
+      if (lowRadix > 1) seq.push_back({which, lowRadix, weight * done, false});
+      seq.push_back({which, 2, weight << cut[i], true});
+      done = int64_t{1} << (cut[i] + 1);
+    }
+    if (extent / done > 1) seq.push_back({which, extent / done, weight * done, false});
+  };
+  for (uint32_t i = 0; i < 2; i++)
+    add(i, a.split[i].numSplit, 1, (int64_t)a.split[i].slabFloor * a.split[i].strideIn, (int64_t)a.split[i].slabFloor * a.split[i].strideOut);
+  int64_t below = 1;
+  for (int k = 0; k < a.mbar.n; k++) {
+    add(2, a.mbar.d[k].extent, below, a.mbar.d[k].strideIn, a.mbar.d[k].strideOut);
+    below *= a.mbar.d[k].extent;
+  }
+  double total = 0;
+  for (const Part& p : seq) total += std::log2((double)p.radix);
+  const double inFlight = std::log2((double)std::max<int64_t>(1, a.itemsPerBlock)) + std::log2((double)std::max<int64_t>(1, residentPerXcd));
+  std::vector<Part> kept, moved;
+  double pos = 0;
+  for (const Part& p : seq) {
+    // (half a digit of margin on the fast side: a digit that only part of the resident workgroups differ in)
+    if (p.bit11 && pos >= inFlight - 0.5 && pos < total - 3.0) moved.push_back(p);
+    else kept.push_back(p);
+    pos += std::log2((double)p.radix);
+  }
+  if (moved.empty() || kept.size() + moved.size() > CUTT_MAX_TILE_DIGITS) return false;
+  std::memset(&dg, 0, sizeof(dg));
+  kept.insert(kept.end(), moved.begin(), moved.end());
+  for (const Part& p : kept) {
+    if (p.radix > 0x7fffffffll || p.weight > 0x7fffffffll) return false;
+    cuttHipTileDigit& o = dg.d[dg.n++];
+    o.which = p.which;
+    o.radix = (uint32_t)p.radix;
+    o.weight = (uint32_t)p.weight;
+    o.div = cuttHipMakeDivisor((uint32_t)p.radix);
+  }
+  return true;
+}
+
 // Fill the launch geometry of a Packed / PackedSplit candidate.  False = does not fit.
 bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptions& opt) {
   const Split& sp = plan.split;
@@ -537,6 +691,20 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
       if (ceilDiv(sp.volMbar, a.itemsPerBlock) * slabs > maxBlocks) a.itemOrder = 0;
     }
   }
+  if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
+  std::memset(&plan.itemDigits, 0, sizeof(plan.itemDigits));
+  if (!opt.itemDigits.empty() && opt.itemOrder < 0) {
+    cuttHipTileDigits dg;
+    // (a text whose radices do not multiply to the extents is ignored)
+    if (parseTileDigits(opt.itemDigits, a.split[0].numSplit, a.split[1].numSplit, sp.volMbar, dg) == items && numberItemsByDigits(a, dg))
+      plan.itemDigits = dg;
+  } else if (opt.addressBits && opt.itemOrder < 0 && a.itemOrder == 0 && opt.xcdAware) {
+    const double cacheBytes = props.infinityCacheBytes > 0 ? (double)props.infinityCacheBytes : 256.0 * 1024 * 1024;
+    cuttHipTileDigits dg;
+    if ((double)pb.volume * pb.elemSize > 0.75 * cacheBytes &&
+        thawAddressBit11(a, pb.elemSize, (int64_t)props.cuCount / kNumXcd * residentPerCU, dg) && numberItemsByDigits(a, dg))
+      plan.itemDigits = dg;
+  }
   const int64_t numbers = cuttHipPackedItemNumbers(&a);
   if (numbers < 1) return false;
   plan.numBlocks = ceilDiv(numbers, a.itemsPerBlock);
@@ -545,7 +713,7 @@ bool setupPacked(Plan& plan, const cuttHipDeviceProps& props, const PlannerOptio
     plan.numBlocks = (int64_t)a.xcdChunk * kNumXcd;
   }
   plan.numThreads = a.numThreads;
-  return fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar);
+  return true;
 }
 
 // Ordering of a tiled launch: fills order, super-tile shape and the per-XCD chunk; returns the
@@ -740,8 +908,12 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
 // of the measuring planner's plan in the mean over all 35 four-rank batched transposes
 // (2^a, 2^j, 2^b, 3) -> (2^b, 2^j, 2^a, 3) of 2e8 8-byte elements (lowest 0.85; the orders it replaces:
 // 0.93 and 0.78), C2 5.6 -> 6.2 TB/s.  With 128 and more tiles along Mk it lost 5-14 % on five of six,
-// so those keep the strips.  Returns the number of logical workgroups, 0 if the tensor is not of
-// this class.
+// so those keep the strips.  The same rule holds with two tiles along an axis and with tile axes over
+// fused ranks (seven such tensors with an Mbar rank between Mm and Mk: +0 ... +11 % against strips and
+// patches, none slower); it does not hold without such a rank, for plain 2-D transposes or with a single
+// tile along an axis (-25 ... +19 %: there one side of a tile is a contiguous stream and the strips that
+// keep it sequential are hard to beat), which is what the caller's conditions exclude.  Returns the
+// number of logical workgroups, 0 if the tensor is not of this class.
 int64_t addressBitOrder(const Problem& pb, const Split& sp, const cuttHipMbar& mb, int64_t tilesM, int64_t tilesK,
                         cuttHipTileDigits& dg) {
   auto log2Exact = [](int64_t v) {
@@ -751,11 +923,26 @@ int64_t addressBitOrder(const Problem& pb, const Split& sp, const cuttHipMbar& m
   };
   const int es = pb.elemSize, esBits = es == 8 ? 3 : 2;
   const int bitsM = log2Exact(tilesM), bitsK = log2Exact(tilesK);
-  if (sp.numMm != 1 || sp.numMk != 1 || bitsM < 2 || bitsK < 2 || tilesK >= 128) return 0;
+  if (bitsM < 1 || bitsK < 1 || tilesK >= 128) return 0;
   if (sp.volMm != tilesM * kTile || sp.volMk != tilesK * kTile) return 0;
-  const int rk = pb.perm[0];
-  const int outM = log2Exact(pb.strideOut[0]), inK = log2Exact(pb.strideIn[rk]);
-  if (outM < 0 || inK < 0) return 0;
+  // A tile axis over fused ranks: its tiles still sit on power-of-two addresses when every rank of the set
+  // has a power-of-two extent and stride; not when the output's next run starts inside the Mm set (those
+  // plans walk strips per Mbar position, tiledBlocks).
+  if (sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm) return 0;
+  // element 2^e of a fused set -> the address bit it moves on the side where the set is not contiguous
+  auto otherBit = [&](int e, bool setIsMm) -> int {
+    int64_t below = 1;
+    const int n = setIsMm ? sp.numMm : sp.numMk;
+    for (int j = 0; j < n; j++) {
+      const int r = setIsMm ? j : pb.perm[j];
+      const int le = log2Exact(pb.dim[r]), ls = log2Exact(setIsMm ? pb.strideOut[r] : pb.strideIn[r]);
+      const int lb = log2Exact(below);
+      if (le < 0 || ls < 0 || lb < 0) return -1;
+      if (e < lb + le) return e - lb + ls + esBits;
+      below *= pb.dim[r];
+    }
+    return -1;
+  };
   struct Digit {
     int which, radix;
     int64_t weight;
@@ -763,8 +950,16 @@ int64_t addressBitOrder(const Problem& pb, const Split& sp, const cuttHipMbar& m
     int index;   // position among the digits of its coordinate
   };
   std::vector<Digit> all;
-  for (int i = 0; i < bitsM; i++) all.push_back({0, 2, int64_t{1} << i, 6 + esBits + i, outM + esBits + 6 + i, i});
-  for (int i = 0; i < bitsK; i++) all.push_back({1, 2, int64_t{1} << i, inK + esBits + 6 + i, 6 + esBits + i, i});
+  for (int i = 0; i < bitsM; i++) {
+    const int wr = otherBit(6 + i, true);
+    if (wr < 0) return 0;
+    all.push_back({0, 2, int64_t{1} << i, 6 + esBits + i, wr, i});
+  }
+  for (int i = 0; i < bitsK; i++) {
+    const int rd = otherBit(6 + i, false);
+    if (rd < 0) return 0;
+    all.push_back({1, 2, int64_t{1} << i, rd, 6 + esBits + i, i});
+  }
   int64_t below = 1;
   int nb = 0, binaryMbar = 0;
   for (int k = 0; k < mb.n; k++) {

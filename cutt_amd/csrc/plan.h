@@ -114,6 +114,7 @@ struct Plan {
   cuttHipTiledArgs tiled;
   cuttHipTiledCopyArgs tcopy;
   cuttHipPackedArgs packed;
+  cuttHipTileDigits itemDigits;  // Packed/PackedSplit: n > 0 if the work items are numbered by these digits (setupPacked)
   size_t ldsBytes = 0;
   int64_t numBlocks = 0;
   int numThreads = 0;
@@ -153,6 +154,9 @@ struct PlannerOptions {
   bool superAuto = true;    // the planner may replace that shape where it measured a better one (see tiledBlocks)
   std::string tileDigits;   // non-empty: tiled order 7 with this mixed-radix numbering, fastest digit first, e.g.
                             // "m2,k8,b0,m0,k0" (m / k = tile along Mm / Mk, b = Mbar position; radix 0 = what is left)
+  std::string itemDigits;   // non-empty: the packed kernel's work items numbered by these digits, same syntax; m / k = slab of
+                            // the first / second cut rank, b = Mbar position; applies to candidates whose slabs are all of one
+                            // size and whose extents the radices multiply to exactly
   bool addressBits = true;  // Tiled: number the workgroups by the address bits their digits move where that rule applies (addressBitOrder)
   int tiledFuse = -1;       // Tiled over fused rank sets: -1 = planner's choice, 0 = one rank per side only
   int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on

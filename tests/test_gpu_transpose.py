@@ -672,3 +672,63 @@ def test_free_tile_numbering(gpu, monkeypatch):
                     info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
                     assert info.tiledOrder == 7
         say("tile digits dim=%s perm=%s done" % (dim, perm))
+
+
+def test_free_item_numbering(gpu, monkeypatch):
+    """The packed kernel's work items numbered by digits (the item number as a mixed-radix number whose digits are
+    dealt out to the slabs of the two cut ranks and the Mbar position): every candidate a digit text applies to,
+    against the oracle, both widths."""
+    import cutt_amd as cutt
+    import oracle
+    dim, perm = (48, 20, 36, 12), (2, 0, 3, 1)
+    for es in (4, 8):
+        data = gpu.seeded(int(np.prod(dim)), es, seed=11 + es)
+        expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
+        ran = 0
+        for digits in ["b2,m0,k0,b0", "b0,k0,m0", "k2,b0,m2,k0,m0", "m0,b3,k0,b0"]:
+            monkeypatch.setenv("CUTT_ITEM_DIGITS", digits)
+            with cutt.Candidates(dim, perm, es) as c:
+                idx = [i for i in range(len(c)) if c.info(i).method_name in ("Packed", "PackedSplit") and c.info(i).tileDigits]
+            for i in idx:
+                info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
+                assert info.tileDigits, (digits, i)
+                ran += 1
+        say("item digits es=%d: %d candidates" % (es, ran))
+        assert ran >= 8
+
+
+def test_address_bit_numberings_at_full_size(gpu):
+    """The numberings the planner derives from address bits, at the sizes where it applies them (beyond the
+    memory-side cache): packed candidates whose bit-11 digit is moved to the top, and Tiled candidates over fused
+    rank sets and with two tiles along an axis numbered by addressBitOrder; against torch's permute on the device."""
+    import torch
+    import cutt_amd as cutt
+    import sweep_runner
+    cases = [((2, 4096, 256, 64), (0, 3, 1, 2), 4, ("Packed", "PackedSplit")),
+             ((128, 256, 8, 128, 8), (2, 3, 0, 1, 4), 4, ("Packed", "PackedSplit")),
+             ((1024, 1024, 128), (2, 1, 0), 8, ("Tiled",)),
+             ((32, 32, 512, 256), (3, 2, 1, 0), 8, ("Tiled",)),
+             ((131072, 8, 4, 32), (3, 2, 1, 0), 8, ("Tiled",))]
+    st = gpu.stream_handle()
+    for dim, perm, es, methods in cases:
+        dim, perm = list(dim), list(perm)
+        vol = int(np.prod(dim, dtype=np.int64))
+        d_in = sweep_runner.index_pattern(vol, es)
+        want = sweep_runner.expected_on_device(d_in, dim, perm)
+        with cutt.Candidates(dim, perm, es) as c:
+            idx = [i for i in range(len(c)) if c.info(i).method_name in methods and c.info(i).tileDigits]
+            best = c.best
+        assert idx, (dim, perm)
+        idx = sorted(idx, key=lambda i: i != best)[:6]
+        for i in idx:
+            d_out = torch.full_like(d_in, -1)
+            rc, h = cutt.cuttPlanFromCandidate(len(dim), dim, perm, es, st, i)
+            assert rc == cutt.CUTT_SUCCESS
+            info = cutt.get_plan_info(h)
+            say("dim=%s perm=%s es=%d candidate %d %s digits %s" % (dim, perm, es, i, info.method_name, info.tileDigits.decode()))
+            assert info.tileDigits
+            assert cutt.cuttExecute(h, d_in.data_ptr(), d_out.data_ptr()) == cutt.CUTT_SUCCESS
+            torch.cuda.synchronize()
+            assert torch.equal(d_out, want), (dim, perm, i)
+            cutt.cuttDestroy(h)
+        del d_in, want

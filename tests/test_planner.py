@@ -315,6 +315,62 @@ def test_free_tile_numbering(cutt, oracle_mod, monkeypatch):
         cutt.set_method_override(0)
 
 
+def test_free_item_numbering(cutt, oracle_mod, monkeypatch):
+    # the packed kernel's work items numbered by digits: the item number as a mixed-radix number whose digits are
+    # dealt out to the slab of the first cut rank (m), of the second (k) and the Mbar position (b).  A text applies
+    # to the candidates whose slabs are of one size and whose extents its radices multiply to; the others keep
+    # their numbering.  Every element exactly once.
+    dim, perm = (24, 10, 18, 6), (2, 0, 3, 1)
+    for digits in ["b2,b3,m0,k0,b0", "m0,k0,b0", "b0,k0,m0", "b3@2,m0,b2@1,k0,b0", "k2,b0,m2,k0,m0"]:
+        monkeypatch.setenv("CUTT_ITEM_DIGITS", digits)
+        with cutt.Candidates(dim, perm, 4, lds_per_block=2048) as c:
+            numbered = [i for i in range(len(c)) if c.info(i).method_name in ("Packed", "PackedSplit") and c.info(i).tileDigits]
+            assert len(numbered) >= 2, (digits, len(numbered))
+            for i in numbered:   # the launch arguments hold one table entry per digit and no slab counts
+                sc = c.data(i, 2)
+                assert sc[8] == 1 and sc[13] == 1 and sc[1] == c.info(i).volMbar * c.info(i).numSplit * c.info(i).numSplit2
+                d = c.data(i, 8)
+                assert len(c.data(i, 0)) == len(d)
+        check_all_candidates(cutt, oracle_mod, dim, perm, 4, need="PackedSplit", lds=2048)
+    # radices that do not multiply to a coordinate's extent, digits of one weight, a digit across two Mbar ranks: ignored
+    for digits in ["b7,m0,k0,b0", "b2@1,b3@1,m0,k0", "b4,b0,m0,k0"]:
+        monkeypatch.setenv("CUTT_ITEM_DIGITS", digits)
+        with cutt.Candidates(dim, perm, 4, lds_per_block=2048) as c:
+            assert all(not c.info(i).tileDigits for i in range(len(c)) if c.info(i).volMbar in (6, 10)), digits
+
+
+def test_packed_items_keep_address_bit_11_moving(cutt, monkeypatch):
+    """Packed plans on power-of-two addresses: a binary digit of the item number that moves the read or the written
+    address by 2 KB (bit 11) and would sit between the digits the resident workgroups differ in and the three
+    slowest ones is taken out of its rank and made the slowest digit."""
+    dim, perm, es = (2, 4096, 256, 64), (0, 3, 1, 2), 4
+    def packed(c):
+        return [i for i in range(len(c)) if c.info(i).method_name in ("Packed", "PackedSplit")]
+    with cutt.Candidates(dim, perm, es) as c:
+        moved = [i for i in packed(c) if c.info(i).tileDigits]
+        assert moved
+        for i in moved:
+            info = c.info(i)
+            d = c.data(i, 8).reshape(-1, 3)          # coordinate, radix, weight
+            assert d[-1][1] == 2                      # the slowest digit is a binary one ...
+            # ... and per coordinate the radices still multiply to the extent
+            ext = [info.numSplit, info.numSplit2, info.volMbar]
+            for w in range(3):
+                assert int(np.prod(d[d[:, 0] == w][:, 1])) == ext[w], (i, d)
+            sc = c.data(i, 2)
+            assert sc[8] == 1 and sc[13] == 1 and sc[1] == ext[0] * ext[1] * ext[2]
+        i = [k for k in moved if c.info(k).numSplit == 256 and c.info(k).numSplit2 == 128][0]
+        # slabs of the second cut rank are 32 elements = 128 bytes apart on the read side: its digit 8 moves bit 11
+        assert c.info(i).tileDigits.decode() == "m256@1,k8@1,k8@16,k2@8"
+    # tensors inside the memory-side cache, extents that are no powers of two, the rule switched off: default numbering
+    for d2, p2 in [((2, 512, 64, 64), (0, 3, 1, 2)), ((2, 4095, 256, 64), (0, 3, 1, 2))]:
+        with cutt.Candidates(d2, p2, es) as c:
+            assert not [i for i in packed(c) if c.info(i).tileDigits], d2
+    monkeypatch.setenv("CUTT_ADDRESS_BITS", "0")
+    with cutt.Candidates(dim, perm, es) as c:
+        assert not [i for i in packed(c) if c.info(i).tileDigits]
+
+
 def test_numbering_by_address_bits(cutt, monkeypatch):
     """Batched transposes on power-of-two addresses: the digits of the workgroup number that move address bit 11
     (on either side) are the three slowest (split over the XCDs), tile digits that move 1 KB / 4 KB and digits
