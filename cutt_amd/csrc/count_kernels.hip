@@ -109,10 +109,8 @@ __device__ __forceinline__ void countAccess(LaneCounts& c, bool write, bool idle
 // functions that kernel uses (tile_order.h: decodeTile, tileLanes, tileReadElem, tileWriteElem).
 template <bool FUSED>
 __global__ __launch_bounds__(kTileThreads) void countTiledKernel(const cuttHipTiledArgs a, unsigned long long* total) {
-  uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
-  uint32_t offIn, offOut;
-  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  uint32_t tm, tk, offIn, offOut;
+  if (!locateTile(a, tm, tk, offIn, offOut)) return;
   const uint32_t es = (uint32_t)a.elemSize, words = es / 4;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const TileLanes t = tileLanes<FUSED>(a, tm, tk, offIn, offOut, lane, wave);
@@ -140,10 +138,8 @@ __global__ __launch_bounds__(kTileThreads) void countTiledKernel(const cuttHipTi
 
 // Mirrors tiledCopyKernel (its whole address arithmetic is the three lines below).
 __global__ __launch_bounds__(kTileThreads) void countTiledCopyKernel(const cuttHipTiledCopyArgs a, unsigned long long* total) {
-  uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
-  uint32_t offIn, offOut;
-  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  uint32_t tm, tk, offIn, offOut;
+  if (!locateTile(a, tm, tk, offIn, offOut)) return;
   const uint32_t es = (uint32_t)a.elemSize;
   const uint32_t lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const uint32_t m0 = tm * kTile, k0 = tk * kTile;

@@ -86,7 +86,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_ITEM_DIGITS", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_ITEM_DIGITS", "CUTT_DIGIT_LANES", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
@@ -425,6 +425,7 @@ PlannerOptions plannerOptions(int forceMethod) {
   if (const char* e = std::getenv("CUTT_TILED_ALIGNED")) opt.tiledAligned = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILE_DIGITS")) opt.tileDigits = e;
   if (const char* e = std::getenv("CUTT_ITEM_DIGITS")) opt.itemDigits = e;
+  if (const char* e = std::getenv("CUTT_DIGIT_LANES")) opt.digitLanes = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_TILED_FUSE")) opt.tiledFuse = std::atoi(e) != 0 ? 1 : 0;
   if (const char* e = std::getenv("CUTT_ADDRESS_BITS")) opt.addressBits = std::atoi(e) != 0;
   return opt;
@@ -1260,6 +1261,17 @@ extern "C" long long cuttCandidatesData(void* list, int index, int what, int cls
             v.push_back(dg.d[k].radix);
             v.push_back(dg.d[k].weight);
           }
+        }
+        break;
+      case 9:  // Tiled / TiledCopy, tile order 7: the digits as the kernels decode them lane-parallel: lanes (0/1), total,
+               // then per digit radix, stepM, stepK, strideIn, strideOut
+        if (p.method != kTiled && p.method != kTiledCopy) return -1;
+        {
+          const cuttHipTileDigits& dg = p.method == kTiled ? p.tiled.digits : p.tcopy.digits;
+          v.push_back(dg.lanes);
+          v.push_back(dg.total);
+          for (int k = 0; k < dg.n && dg.lanes; k++)
+            v.insert(v.end(), {dg.lane[k].radix, dg.lane[k].stepM, dg.lane[k].stepK, dg.lane[k].strideIn, dg.lane[k].strideOut});
         }
         break;
       default:

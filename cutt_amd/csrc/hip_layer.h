@@ -109,10 +109,28 @@ typedef struct cuttHipTileDigit {
   cuttHipDivisor div;   /* division by radix (cuttHipMakeDivisor) */
 } cuttHipTileDigit;
 
+/* One digit as the kernels decode it: lane i of a wavefront takes digit i, computes its value
+ * (index / below) % radix with two multiply-high divisions (constants as in cuttHipMbarDim) and
+ * contributes value * step to the tile coordinates and to the two offsets of the Mbar position. */
+typedef struct cuttHipDigitLane {
+  uint32_t belowMul, radixMul, ctl, radix;
+  uint32_t stepM, stepK;          /* tiles along Mm / Mk per unit of the digit (its weight, or 0) */
+  uint32_t strideIn, strideOut;   /* elements per unit of an Mbar digit on the two sides (or 0) */
+} cuttHipDigitLane;
+
 typedef struct cuttHipTileDigits {
   int n;
   cuttHipTileDigit d[CUTT_MAX_TILE_DIGITS];
+  /* Filled by cuttHipFinishTileDigits from d[] and the plan's Mbar table.  lanes = 1 if every Mbar
+   * digit stays inside one Mbar rank, so that the offsets are linear in the digits: the kernels then
+   * decode a workgroup index with lane[] in one step; otherwise (lanes = 0) digit by digit. */
+  int lanes;
+  uint32_t total;                 /* product of the radices: indices from here on are padding */
+  cuttHipDigitLane lane[CUTT_MAX_TILE_DIGITS];
 } cuttHipTileDigits;
+/* Derive lanes, total and lane[] of a digit list from d[] and the Mbar table of the same plan
+ * (returns 0; a list that cannot be decoded in one step gets lanes = 0). */
+int cuttHipFinishTileDigits(cuttHipTileDigits* dg, const cuttHipMbar* mb);
 
 /*
  * Offsets of the rows of a tile when a tile axis runs over several fused ranks: row index i along the

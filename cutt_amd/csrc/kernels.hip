@@ -34,6 +34,7 @@
 
 #include <algorithm>
 #include <atomic>
+#include <cstring>
 #include <mutex>
 #include <tuple>
 #include <type_traits>
@@ -86,10 +87,8 @@ __global__ __launch_bounds__(kTileThreads) void tiledKernel(const cuttHipTiledAr
                                                             T* __restrict__ out) {
   __shared__ T tile[kTile][kTile + 1];
 
-  uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
-  uint32_t offIn, offOut;
-  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  uint32_t tm, tk, offIn, offOut;
+  if (!locateTile(a, tm, tk, offIn, offOut)) return;
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -182,10 +181,8 @@ __global__ __launch_bounds__(kTileThreads) void tiledAlignedKernel(const cuttHip
   constexpr int RD = (ROWS + kWaves - 1) / kWaves;  // rows a wave reads at most
   __shared__ T tile[ROWS][kTile + 1];
 
-  uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
-  uint32_t offIn, offOut;
-  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  uint32_t tm, tk, offIn, offOut;
+  if (!locateTile(a, tm, tk, offIn, offOut)) return;
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -261,10 +258,8 @@ template <typename T, int NT>
 __global__ __launch_bounds__(kTileThreads) void tiledCopyKernel(const cuttHipTiledCopyArgs a,
                                                                 const T* __restrict__ in,
                                                                 T* __restrict__ out) {
-  uint32_t tm, tk, m;
-  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return;
-  uint32_t offIn, offOut;
-  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  uint32_t tm, tk, offIn, offOut;
+  if (!locateTile(a, tm, tk, offIn, offOut)) return;
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -450,7 +445,7 @@ bool divisorOk(const cuttHipDivisor& dv, uint32_t d) {
 
 // Number of workgroups of a tiled launch; checks the ordering parameters.
 bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk, uint32_t superM,
-              uint32_t superK, const cuttHipTileDigits& dg, uint64_t& blocks) {
+              uint32_t superK, const cuttHipTileDigits& dg, const cuttHipMbar& mbar, uint64_t& blocks) {
   uint64_t logical = (uint64_t)tilesM * tilesK * (uint64_t)volMbar;
   if (order == 7) {
     if (dg.n < 1 || dg.n > CUTT_MAX_TILE_DIGITS) return false;
@@ -476,6 +471,14 @@ bool tileGrid(int order, int tilesM, int tilesK, int volMbar, uint32_t xcdChunk,
       for (int i = 0; i < dg.n; i++)
         if (dg.d[i].which == w && dg.d[i].radix > 1) all *= dg.d[i].radix;
       if (span != all || span < extent[w]) return false;
+    }
+    // what the kernels decode with must be what cuttHipFinishTileDigits derives from the list
+    // (a list without lanes is decoded digit by digit, which needs none of this)
+    if (dg.lanes) {
+      cuttHipTileDigits want = dg;
+      if (cuttHipFinishTileDigits(&want, &mbar) != 0 || want.lanes != 1 || want.total != dg.total ||
+          std::memcmp(want.lane, dg.lane, sizeof(dg.lane)) != 0)
+        return false;
     }
   } else if (order >= 3) {
     if (superM < 1 || superK < 1) return false;
@@ -583,14 +586,14 @@ hipError_t launchKernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t 
 
 extern "C" long long cuttHipTiledGrid(const cuttHipTiledArgs* a) {
   uint64_t blocks = 0;
-  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return 0;
   return (long long)blocks;
 }
 
 extern "C" long long cuttHipTiledCopyGrid(const cuttHipTiledCopyArgs* a) {
   uint64_t blocks = 0;
-  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!a || !tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return 0;
   return (long long)blocks;
 }
@@ -605,7 +608,7 @@ extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
       (a->alignedStores && (a->rowsK.n > 0 || a->rowsM.n > 0)))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   return 0;
@@ -614,7 +617,7 @@ extern "C" int cuttHipValidateTiled(const cuttHipTiledArgs* a) {
 extern "C" int cuttHipLaunchTiled(const cuttHipTiledArgs* a, const void* in, void* out, void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);
@@ -649,7 +652,7 @@ extern "C" int cuttHipValidateTiledCopy(const cuttHipTiledCopyArgs* a) {
       a->order < 0 || a->order > 7 || !mbarOk(a->mbar))
     return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return (int)hipErrorInvalidConfiguration;
   if (a->cachePolicy != 0 && a->cachePolicy != 1 && a->cachePolicy != 3) return (int)hipErrorInvalidValue;
   return 0;
@@ -659,7 +662,7 @@ extern "C" int cuttHipLaunchTiledCopy(const cuttHipTiledCopyArgs* a, const void*
                                       void* stream) {
   if (!a || !in || !out) return (int)hipErrorInvalidValue;
   uint64_t blocks = 0;
-  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, blocks))
+  if (!tileGrid(a->order, a->tilesM, a->tilesK, a->volMbar, a->xcdChunk, a->superM, a->superK, a->digits, a->mbar, blocks))
     return (int)hipErrorInvalidConfiguration;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((uint32_t)blocks), block(kTileThreads);

@@ -43,6 +43,59 @@ extern "C" int cuttHipFinishMbar(cuttHipMbar* mb) {
   return 0;
 }
 
+static int finishTileDigits(cuttHipTileDigits* dg, const cuttHipMbar* mb);
+
+extern "C" int cuttHipFinishTileDigits(cuttHipTileDigits* dg, const cuttHipMbar* mb) {
+  if (!dg || !mb) return -1;
+  finishTileDigits(dg, mb);
+  if (!dg->lanes) {  // not decodable in one step: no half-filled table
+    dg->total = 0;
+    for (int i = 0; i < CUTT_MAX_TILE_DIGITS; i++) dg->lane[i] = cuttHipDigitLane{0u, 0u, 0u, 1u, 0u, 0u, 0u, 0u};
+  }
+  return 0;
+}
+
+static int finishTileDigits(cuttHipTileDigits* dg, const cuttHipMbar* mb) {
+  dg->lanes = 0;
+  dg->total = 0;
+  for (int i = 0; i < CUTT_MAX_TILE_DIGITS; i++) dg->lane[i] = cuttHipDigitLane{0u, 0u, 0u, 1u, 0u, 0u, 0u, 0u};
+  if (dg->n < 1 || dg->n > CUTT_MAX_TILE_DIGITS || mb->n < 0 || mb->n > CUTT_MAX_RANK) return 0;
+  uint64_t below = 1, mbarDigits = 1, volMbar = 1;
+  for (int k = 0; k < mb->n; k++) volMbar *= mb->d[k].extent;
+  for (int i = 0; i < dg->n; i++) {
+    const cuttHipTileDigit& d = dg->d[i];
+    cuttHipDigitLane& l = dg->lane[i];
+    if (d.radix < 1 || d.which > 2 || below * d.radix >= (1ull << 31)) return 0;
+    const cuttHipDivisor b = cuttHipMakeDivisor((uint32_t)below), e = cuttHipMakeDivisor(d.radix);
+    l.belowMul = b.mul;
+    l.radixMul = e.mul;
+    l.ctl = b.shift | (e.shift << 8) | (b.add << 16) | (e.add << 17);
+    l.radix = d.radix;
+    if (d.which == 0) l.stepM = d.weight;
+    if (d.which == 1) l.stepK = d.weight;
+    if (d.which == 2 && d.radix > 1) {
+      // the Mbar rank the digit counts in; it must not reach into the next one
+      uint64_t rankBelow = 1;
+      int k = 0;
+      for (; k < mb->n; rankBelow *= mb->d[k].extent, k++)
+        if ((uint64_t)d.weight >= rankBelow && (uint64_t)d.weight < rankBelow * mb->d[k].extent) break;
+      if (k == mb->n || (uint64_t)d.weight % rankBelow != 0) return 0;
+      const uint64_t u = (uint64_t)d.weight / rankBelow;
+      if ((uint64_t)mb->d[k].extent % (u * d.radix) != 0) return 0;
+      mbarDigits *= d.radix;
+      if (u * mb->d[k].strideIn > 0xffffffffull || u * mb->d[k].strideOut > 0xffffffffull) return 0;
+      l.strideIn = (uint32_t)(u * mb->d[k].strideIn);
+      l.strideOut = (uint32_t)(u * mb->d[k].strideOut);
+    }
+    below *= d.radix;
+  }
+  // (no Mbar position beyond the last one: the kernels do not rebuild the position to check it)
+  if (mbarDigits != volMbar) return 0;
+  dg->total = (uint32_t)below;
+  dg->lanes = 1;
+  return 0;
+}
+
 extern "C" long long cuttHipPackedItemNumbers(const cuttHipPackedArgs* a) {
   const unsigned long long slabs = (unsigned long long)a->split[0].numSplit * (unsigned long long)a->split[1].numSplit;
   unsigned long long n = (unsigned long long)a->volMbar * slabs;

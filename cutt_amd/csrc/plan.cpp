@@ -1093,6 +1093,14 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
                                    sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm, o, a.digits);
     }
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
+    // How the kernels decode a free numbering.  Digit by digit costs a chain of up to 16 dependent scalar loads
+    // per workgroup, which a workgroup that moves a full tile hides but one that moves a quarter of it does not
+    // (a (4194304,32) transpose of 4-byte elements in the digits of its default order: 4.4 TB/s digit by digit,
+    // 5.8 TB/s with one digit per lane, 5.6-5.7 TB/s in the default order itself; 8-byte elements 5.1 / 5.4 /
+    // 5.5).  On full tiles of 8-byte elements the lane-parallel decode is the slower one by 1-2 % (C2 6.13
+    // against 6.21 TB/s, four of seven such plans; the others equal), so it is used for tiles of at most 8 KB.
+    const int64_t tileBytes = std::min<int64_t>(sp.volMm, kTile) * std::min<int64_t>(sp.volMk, kTile) * pb.elemSize;
+    if (a.order == 7 && (opt.digitLanes > 0 || (opt.digitLanes < 0 && tileBytes <= 8192))) cuttHipFinishTileDigits(&a.digits, &a.mbar);
     a.cachePolicy = opt.cachePolicy;
     a.grouped = opt.tiledGrouped > 0 && !a.alignedStores ? 1 : 0;  // -1: decided from the model's estimate later
     plan.ldsBytes = (size_t)(kTile + (a.alignedStores ? 128 / pb.elemSize - 1 : 0)) * (kTile + 1) * pb.elemSize;
@@ -1115,6 +1123,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
+    if (a.order == 7 && opt.digitLanes > 0) cuttHipFinishTileDigits(&a.digits, &a.mbar);
     plan.ldsBytes = 0;
   }
   plan.numThreads = 256;

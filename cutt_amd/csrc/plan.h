@@ -157,6 +157,7 @@ struct PlannerOptions {
   std::string itemDigits;   // non-empty: the packed kernel's work items numbered by these digits, same syntax; m / k = slab of
                             // the first / second cut rank, b = Mbar position; applies to candidates whose slabs are all of one
                             // size and whose extents the radices multiply to exactly
+  int digitLanes = -1;      // tile order 7: decode the digits lane-parallel (1), digit by digit (0), planner's choice (-1)
   bool addressBits = true;  // Tiled: number the workgroups by the address bits their digits move where that rule applies (addressBitOrder)
   int tiledFuse = -1;       // Tiled over fused rank sets: -1 = planner's choice, 0 = one rank per side only
   int tiledAligned = -1;    // Tiled: line-aligned stores, -1 = planner's choice, 0 = off, 1 = on

@@ -112,6 +112,33 @@ __device__ __forceinline__ bool decodeTile(uint32_t bid, const TileOrder o, uint
   return m < volMbar && tm < tilesM && tk < tilesK;
 }
 
+// Workgroup index -> tile coordinates and the offsets of its Mbar position (all wave-uniform); false for
+// a padding workgroup.  With a digit list that the host could turn into lanes (cuttHipFinishTileDigits)
+// lane i of every row of 16 lanes takes digit i - two multiply-high divisions give its value - and four row
+// sums add up what the digits contribute; nothing is read digit by digit.  Otherwise decodeTile and the
+// Mbar table.
+template <typename Args>
+__device__ __forceinline__ bool locateTile(const Args& a, uint32_t& tm, uint32_t& tk, uint32_t& offIn, uint32_t& offOut) {
+  if (a.order == 7 && a.digits.lanes) {
+    const uint32_t l = a.xcdChunk ? (blockIdx.x % kNumXcd) * a.xcdChunk + blockIdx.x / kNumXcd : blockIdx.x;
+    if (l >= a.digits.total) return false;
+    static_assert(CUTT_MAX_TILE_DIGITS == 16, "one DPP row of 16 lanes holds the digits");
+    const cuttHipDigitLane d = a.digits.lane[threadIdx.x & 15];  // (entries beyond the list contribute 0)
+    const uint32_t q = fastDivide(l, d.belowMul, d.ctl & 0xff, (d.ctl >> 16) & 1);
+    const uint32_t q2 = fastDivide(q, d.radixMul, (d.ctl >> 8) & 0xff, (d.ctl >> 17) & 1);
+    const uint32_t v = q - q2 * d.radix;
+    tm = (uint32_t)__builtin_amdgcn_readfirstlane((int)rowSum(v * d.stepM));
+    tk = (uint32_t)__builtin_amdgcn_readfirstlane((int)rowSum(v * d.stepK));
+    offIn = (uint32_t)__builtin_amdgcn_readfirstlane((int)rowSum(v * d.strideIn));
+    offOut = (uint32_t)__builtin_amdgcn_readfirstlane((int)rowSum(v * d.strideOut));
+    return tm < (uint32_t)a.tilesM && tk < (uint32_t)a.tilesK;
+  }
+  uint32_t m;
+  if (!decodeTile(blockIdx.x, TileOrder{a.order, a.xcdChunk, a.superM, a.superK, &a.digits}, a.tilesM, a.tilesK, a.volMbar, tm, tk, m)) return false;
+  mbarOffsets(loadMbarLane(a.mbar, threadIdx.x & 63), m, offIn, offOut);
+  return true;
+}
+
 // Offset of row `i` of a tile axis that runs over the fused ranks of `rr` (rr.n >= 1), per lane.
 __device__ __forceinline__ uint32_t rowOffset(const cuttHipRowRadix& rr, uint32_t i) {
   uint32_t off = 0;

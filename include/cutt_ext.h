@@ -182,6 +182,12 @@ long long cuttSlabDecomposition(int rank, const int* dim, const int* permutation
  *   what 3: class scalars: vol, inCont, outCont
  *   what 4: rowIn[] (vol/inCont input offsets, one per contiguous run)
  *   what 5: rowOut[] (vol/outCont output offsets)   what 6: shIdx[] (vol LDS gather slots)
+ *   what 7: Tiled over fused rank sets: (extent, stride) of the ranks a tile axis runs over (cls 0 = Mk, 1 = Mm)
+ *   what 8: the digits of a free numbering (tile order 7, or a packed plan's work items), fastest first:
+ *           (coordinate, radix, weight) each
+ *   what 9: tile order 7, the same digits as the kernels decode them with one digit per lane: lanes (1 if
+ *           the list allows that), the product of the radices, then per digit (radix, tiles along Mm and
+ *           along Mk per unit, input and output offset per unit)
  */
 long long cuttCandidatesData(void* list, int index, int what, int cls, long long* values,
                              long long maxCount);

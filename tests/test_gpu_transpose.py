@@ -659,19 +659,28 @@ def test_free_tile_numbering(gpu, monkeypatch):
     import oracle
     cases = [((200, 6, 300, 3), (2, 1, 0, 3)), ((70, 130), (1, 0)), ((650, 3, 5, 70), (3, 1, 2, 0)), ((150, 7, 300), (0, 2, 1)),
              ((512, 12, 512, 3), (2, 1, 0, 3))]
+    seen_lanes = 0
     for dim, perm in cases:
         for es in (4, 8):
             data = gpu.seeded(int(np.prod(dim)), es, seed=3 + es)
             expect = oracle.transpose_mt(list(dim), list(perm), data, 8)
-            for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0", "m2@2,b2@2,m2@1,k0,b2@1,b0,m0"]:
-                monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
-                with cutt.Candidates(dim, perm, es) as c:
-                    idx = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]
-                assert idx
-                for i in idx:
-                    info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
-                    assert info.tiledOrder == 7
+            # both decoders of the kernels: digit by digit, and one digit per lane (which the library falls back from
+            # where an Mbar digit runs over two ranks or the digits overshoot the Mbar extent)
+            for lanes in ("0", "1"):
+                monkeypatch.setenv("CUTT_DIGIT_LANES", lanes)
+                for digits in ["m2,k8,b0,m0,k0", "b4,k2,m0,b0,k0", "k0,m0,b0", "m3,k3,b5,m3,k3,b0,m0,k0", "b0", "m2@2,b2@2,m2@1,k0,b2@1,b0,m0",
+                               "m2,k8,b2,b3,m0,k0,b0", "b3,k2,m0,b2,k0,b0"]:
+                    monkeypatch.setenv("CUTT_TILE_DIGITS", digits)
+                    with cutt.Candidates(dim, perm, es) as c:
+                        idx = [i for i in range(len(c)) if c.info(i).method_name in ("Tiled", "TiledCopy")]
+                        one_per_lane = sum(int(c.data(i, 9)[0]) for i in idx)
+                    assert idx
+                    seen_lanes += one_per_lane
+                    for i in idx:
+                        info = gpu.check_case(list(dim), list(perm), es, data=data, how="candidate", candidate=i, expect=expect)
+                        assert info.tiledOrder == 7
         say("tile digits dim=%s perm=%s done" % (dim, perm))
+    assert seen_lanes >= 20   # the second decoder did run
 
 
 def test_free_item_numbering(gpu, monkeypatch):

@@ -315,6 +315,55 @@ def test_free_tile_numbering(cutt, oracle_mod, monkeypatch):
         cutt.set_method_override(0)
 
 
+def test_digits_one_per_lane_decode_like_digit_by_digit(cutt, monkeypatch):
+    """Tile order 7 has two decoders in the kernels: digit by digit, and - where every Mbar digit stays inside one
+    Mbar rank - one digit per lane, whose contributions (tile coordinates, offsets of the Mbar position) add up.
+    The table the second one reads must give, for every workgroup index, what the first one gives."""
+    monkeypatch.setenv("CUTT_DIGIT_LANES", "1")
+    cutt.set_method_override(4)
+    try:
+        cases = [((256, 6, 4, 320), (3, 1, 2, 0), "m2,b2,k0,b3,b4,m0"), ((256, 6, 4, 320), (3, 1, 2, 0), "b6@1,k0,m0,b4@6"),
+                 ((128, 8, 192), (2, 1, 0), "k3,b2@4,m0,b4@1"), ((200, 6, 300, 3), (2, 1, 0, 3), "m2,k8,b6,b3,m0,k0"),
+                 ((200, 6, 300, 3), (2, 1, 0, 3), "m2,k8,b0,m0,k0")]   # the last one: an Mbar digit over two ranks, no lanes
+        with_lanes = 0
+        for dim, perm, text in cases:
+            monkeypatch.setenv("CUTT_TILE_DIGITS", text)
+            with cutt.Candidates(dim, perm, 8) as c:
+                i = [k for k in range(len(c)) if c.info(k).method_name == "Tiled" and c.info(k).numMm == 1 and c.info(k).numMk == 1][0]
+                assert c.info(i).tiledOrder == 7
+                digits = c.data(i, 8).reshape(-1, 3)
+                lanes = c.data(i, 9)
+                mbar = c.data(i, 0).reshape(-1, 3)
+                if text.endswith("b0,m0,k0"):
+                    assert lanes[0] == 0
+                    continue
+                assert lanes[0] == 1 and lanes[1] == int(np.prod(digits[:, 1]))
+                with_lanes += 1
+                table = lanes[2:].reshape(-1, 5)
+                vol_mbar = int(np.prod(mbar[:, 0])) if len(mbar) else 1
+                for l in range(int(lanes[1])):
+                    rest, coord = l, [0, 0, 0]
+                    for which, radix, weight in digits:
+                        rest, v = divmod(rest, int(radix))
+                        coord[which] += v * int(weight)
+                    assert coord[2] < vol_mbar
+                    off_in = off_out = 0
+                    m = coord[2]
+                    for e, si, so in mbar:
+                        m, idx = divmod(m, int(e))
+                        off_in += idx * int(si)
+                        off_out += idx * int(so)
+                    got, below = [0, 0, 0, 0], 1
+                    for radix, step_m, step_k, si, so in table:
+                        v = (l // below) % int(radix)
+                        below *= int(radix)
+                        got = [got[0] + v * int(step_m), got[1] + v * int(step_k), got[2] + v * int(si), got[3] + v * int(so)]
+                    assert got == [coord[0], coord[1], off_in, off_out], (text, l)
+        assert with_lanes == 4
+    finally:
+        cutt.set_method_override(0)
+
+
 def test_free_item_numbering(cutt, oracle_mod, monkeypatch):
     # the packed kernel's work items numbered by digits: the item number as a mixed-radix number whose digits are
     # dealt out to the slab of the first cut rank (m), of the second (k) and the Mbar position (b).  A text applies
