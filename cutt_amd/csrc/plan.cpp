@@ -822,29 +822,27 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   if (opt.superAuto && o.order == 5) {
     // Strips that run through all of Mk keep the tiles that share a partly covered line close
     // together.  When all rows start and end on the 128-byte grid on both sides no line is shared
-    // between tiles, and patches that are short along Mk bring the next Mbar position (usually the
-    // neighbouring rows in memory) back sooner.  Measured on forced Tiled plans of 6e7-2.6e8
-    // 8-byte elements, every shape timed: patches of 8 tiles along Mk, 4 tiles wide when both
-    // ranks have 16 tiles and more, ran +2.5 % in the mean over 14 random such tensors (-1.7 %
+    // between tiles, and patches that are short along Mk bring the next Mbar position back sooner, which
+    // pays when that position is the neighbouring row of the same matrix on both sides (an Mbar rank
+    // between Mm and Mk).  Measured on forced Tiled plans of 6e7-2.6e8 8-byte elements, every shape
+    // timed: patches of 8 tiles along Mk ran +2.5 % in the mean over 14 random such tensors (-1.7 %
     // ... +9 %) and +2...+6 % on five batched transposes of 1024 x 1024-like matrices with rows up
-    // to 512 KB apart.  Outside these limits it loses: 4-byte elements -3 % (worst -16 %), rows
-    // off the grid -7 %, 10 tiles along Mk cut into 5 + 5 -1...-6 %, fewer than three tiles along
-    // Mm -2 %.
-    // Re-measured later, four against two tiles wide where Mm has 16 tiles and more: two wide gained
-    // +0.9 ... +5.7 % on five of six batched transposes of 1024 x 1024-like matrices with an Mbar rank
-    // between the two (C2: 5.53 -> 5.61 TB/s; one -2 %) and +1.3 % in the mean over twelve random tensors
-    // on the grid (-0.8 ... +5.5 %).  Two wide from 8 tiles on, or patches when Mk has exactly 8 tiles,
-    // did not hold up on random tensors (-1 ... -6 % on five of seven; -11 % on (768,64,512,3)/(2,0,1,3)).
+    // to 512 KB apart; two instead of eight tiles wide where Mm has 16 tiles and more gained another
+    // +0.9 ... +5.7 % on five of six of the latter (one -2 %).  Outside these limits it loses: 4-byte
+    // elements -3 % (worst -16 %), rows off the grid -7 %, 10 tiles along Mk cut into 5 + 5 -1...-6 %,
+    // fewer than three tiles along Mm -2 %.
+    // Checked again on tensors the rule was not found on (70 seeded plans with extents that are
+    // multiples of 16, patches against strips in one process): with the rank between +1 % in the mean
+    // over 27 (-7 ... +9 %; +4 % over ten batched transposes whose extents are multiples of 256), for
+    // batches of separate matrices - the Mbar rank slowest on both sides, which used to get 8 x 8
+    // patches - -1.3 % over 20 (-7 ... +3 %): those walk strips again.
     const bool onGrid = rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0;
-    gridRule = onGrid && elemSize == 8 && tilesK >= 16 && tilesM >= 3;
+    gridRule = onGrid && elemSize == 8 && tilesK >= 16 && tilesM >= 3 && mbarBetween;
     if (gridRule) {
       superK = 8;
-      // (Two wide only when an Mbar rank lies between Mm and Mk on both sides, as in C2: there the next Mbar
-      // position is the neighbouring row of the same patch.  Batches of separate matrices ran 5 % faster
-      // with patches 8 x 8 than 2 x 8 - twenty random ones, -1 ... +23 % - and tensors with the rank between
-      // were unchanged by the distinction.  Nor for input rows a multiple of 32 KB apart, see below: ten such
-      // tensors with the rank between ran 3.4 % faster 8 wide, -0.6 ... +7 %.)
-      if (tilesM >= 16 && mbarBetween && rowBytesIn % 32768 != 0) superM = 2;
+      // (Not two wide for input rows a multiple of 32 KB apart: ten such tensors ran 3.4 % faster 8 wide,
+      // -0.6 ... +7 %.)
+      if (tilesM >= 16 && rowBytesIn % 32768 != 0) superM = 2;
     }
   }
   if (opt.superAuto && (o.order == 5 || o.order == 3) && elemSize == 4 && beyondCache && rowBytesIn > 0 &&
