@@ -858,10 +858,11 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
     gridRule = true;
     superM = 16;
   }
-  if (opt.superAuto && !gridRule && (o.order == 5 || o.order == 3) && tilesM > superM && tilesM <= 16 &&
+  if (opt.superAuto && !gridRule && (o.order == 5 || o.order == 3) && tilesM > superM && tilesM <= 14 &&
       !(elemSize == 8 && rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0)) {
-    // A rank of 9..16 tiles is not cut into two strips (5 + 4 ... 8 + 8): one strip as wide as the rank
-    // reads whole input rows.  Forced Tiled plans on 13 random tensors with such a rank (both widths,
+    // A rank of 9..14 tiles is not cut into two strips (5 + 4 ... 7 + 7): one strip as wide as the rank
+    // reads whole input rows.  (Up to 16 tiles at first; on 32 seeded tensors the rule was not found on, the
+    // seven with 15 or 16 tiles all ran slower in one strip, -0.6 ... -9 %, the others +3 % in the mean.)  Forced Tiled plans on 13 random tensors with such a rank (both widths,
     // with and without Mbar ranks): +2.8 % in the mean, -2 % ... +8 %; the three-rank reversals of the
     // reference's bench 5 with 13 tiles along Mm and 3 along Mk, (817,1480,148)-like: 749 -> 660 us.
     // From 17 tiles on a single strip gains nothing in the mean (-7 % ... +9 %) and stays cut.  Not for

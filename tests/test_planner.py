@@ -212,7 +212,8 @@ def test_super_tile_shapes_of_the_tiled_plan(cutt):
     assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 8) == (7, 1, 1)
     assert tiled((2048, 1024, 95), (1, 0, 2), 8) == (5, 8, 16)      # a batch of separate matrices: strips
     assert tiled((4096, 12, 3936), (2, 1, 0), 8) == (5, 8, 8)       # input rows a multiple of 32 KB
-    assert tiled((1000, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 16, 16)   # 4-byte: one strip for a rank of 16 tiles
+    assert tiled((850, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 14, 16)    # 4-byte: one strip for a rank of 14 tiles
+    assert tiled((1000, 64, 1024, 3), (2, 1, 0, 3), 4) == (5, 8, 16)    # ... two for 16
     assert tiled((1024, 64, 1024, 3), (2, 1, 0, 3), 4) == (7, 1, 1)
     # 4-byte input rows a multiple of 32 KB apart: strips 16 wide, beyond the memory-side cache only
     assert tiled((8192, 8192), (1, 0), 4) == (3, 16, 128)
