@@ -1,5 +1,5 @@
 // Host-side stress of the planner for the sanitizer tests: four caller threads put random
-// problems (ranks 2-7, both element sizes) through the candidate API, which enumerates the
+// problems (ranks 2-7, both element sizes, every fourth one with power-of-two extents) through the candidate API, which enumerates the
 // candidates, builds their index tables and runs the cost model on the planner's own helper
 // threads.  Needs no GPU.  Prints "done, refused N".
 #include <cmath>
@@ -22,6 +22,13 @@ static int work(unsigned seed, int count) {
     for (int r = 0; r < rank; r++) {
       dim[r] = 2 + (int)(rng() % (unsigned)(2 * mean));
       perm[r] = r;
+    }
+    if (it % 4 == 3) {
+      // every fourth problem: extents that are powers of two, 2^26-2^28 elements - the tensors on which the
+      // planner numbers workgroups and work items by address bits
+      int bits = 26 + (int)(rng() % 3);
+      for (int r = 0; r < rank; r++) dim[r] = 2;
+      for (bits -= rank; bits > 0; bits--) dim[rng() % (unsigned)rank] *= 2;
     }
     for (int r = rank - 1; r > 0; r--) std::swap(perm[r], perm[rng() % (unsigned)(r + 1)]);
     void* list = cuttCandidatesCreate(rank, dim.data(), perm.data(), (rng() & 1) ? 4 : 8);
