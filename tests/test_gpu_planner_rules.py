@@ -237,6 +237,29 @@ def test_thin_second_tile_lets_the_tiles_along_mk_run_fastest():
              1.0, 0.93, 3)
 
 
+def test_output_rows_front_to_back_for_matrices_on_the_line_grid():
+    # matrices and batches of separate matrices with extents that are multiples of 64, 17-700 tiles along Mk and 16
+    # and more along Mm: the tiles along Mk run fastest instead of strips (found: +4 % in the mean over 90 such
+    # plans of three seeded sets, most between -2 and +9 %)
+    rng = np.random.default_rng(2718)
+    cases = []
+    while len(cases) < 16:
+        es = 4 if len(cases) % 2 == 0 else 8
+        batch = 1 if len(cases) % 4 < 2 else int(rng.integers(2, 7))
+        total = 2.0 ** rng.uniform(26.2, 28.2) * 4 / es / batch
+        n = 64 * int(rng.integers(17, 500))
+        m = int(total / n) // 64 * 64
+        row = m * es
+        if m < 1024 or row % 4096 == 0 or not (1024 <= row % 16384 <= 16384 - 1024):
+            continue
+        cases.append(dict(dim=(m, n) if batch == 1 else (m, n, batch), perm=(1, 0) if batch == 1 else (1, 0, 2), es=es))
+    plain = [c for c in cases if len(c["dim"]) == 2]
+    batched = [c for c in cases if len(c["dim"]) == 3]
+    used = lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.tiledOrder == 2 and off.tiledOrder != 2
+    run_rule("output rows front to back (matrices)", plain, {"CUTT_TILED_ORDER": "3"}, used, 1.01, 0.93, 5)
+    run_rule("output rows front to back (batches)", batched, {"CUTT_TILED_ORDER": "5"}, used, 1.01, 0.93, 5)
+
+
 def test_work_items_per_workgroup_and_their_order():
     # packed plans: the planner's items per workgroup (two for 8-byte blocks of 10 KB and more, else four) against
     # four always, and the order in which a workgroup takes its items (its own slabs at several Mbar positions

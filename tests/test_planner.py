@@ -221,6 +221,17 @@ def test_super_tile_shapes_of_the_tiled_plan(cutt):
     assert tiled((8192, 2048), (1, 0), 4) == (3, 8, 32)
     assert tiled((4096, 16384), (1, 0), 4) == (3, 8, 256)
     assert tiled((8192, 8192), (1, 0), 8) == (3, 8, 128)
+    # matrices with all rows on the line grid: the tiles along Mk run fastest (order 2) with 17-700 tiles there ...
+    assert tiled((45440, 4416), (1, 0), 4)[0] == 2
+    assert tiled((10112, 11712, 2), (1, 0, 2), 8)[0] == 2
+    assert tiled((45440, 1024), (1, 0), 8)[0] == 3        # ... 16 tiles along Mk: strips
+    assert tiled((2816, 51200), (1, 0), 4)[0] == 3        # 800 tiles
+    assert tiled((45441, 4416), (1, 0), 4)[0] == 3        # rows off the line grid
+    assert tiled((20480, 3392), (1, 0), 8)[0] == 3        # input rows a multiple of 4 KB apart
+    assert tiled((8256, 16896), (1, 0), 4)[0] == 3        # ... and within 1 KB of a multiple of 16 KB
+    assert tiled((4416, 25856), (1, 0), 4)[0] == 2
+    assert tiled((4416, 8, 12928), (2, 1, 0), 4)[0] == 5     # an Mbar rank between Mm and Mk: not this rule
+    assert tiled((2240, 2752), (1, 0), 8)[0] == 3         # inside the memory-side cache
 
 
 def test_every_tile_order_visits_every_tile_once(cutt, oracle_mod, monkeypatch):
