@@ -86,7 +86,7 @@ std::string planKey(int deviceID, int force, int rank, const int* dim, const int
   for (int i = 0; i < rank; i++) put(perm[i]);
   for (const char* name : {"CUTT_TILED_ORDER", "CUTT_XCD_AWARE", "CUTT_ELEMS_PER_THREAD", "CUTT_PACKED_ROUNDS",
                            "CUTT_MAX_ITEMS", "CUTT_ITEM_ORDER", "CUTT_PAD_SHIFT", "CUTT_CACHE_POLICY", "CUTT_WIDE_OFFSETS", "CUTT_MBAR_ORDER",
-                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_ITEM_DIGITS", "CUTT_DIGIT_LANES", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS"}) {
+                           "CUTT_SUPER_M", "CUTT_SUPER_K", "CUTT_TILED_GROUPED", "CUTT_TILED_ALIGNED", "CUTT_TILE_DIGITS", "CUTT_ITEM_DIGITS", "CUTT_DIGIT_LANES", "CUTT_TILED_FUSE", "CUTT_ADDRESS_BITS", "CUTT_MODEL_RUN_LENGTH"}) {
     const char* e = std::getenv(name);
     k += e ? e : "-";
     k += ';';
