@@ -806,6 +806,13 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   // reference's suites whose fused-Mm plan has one or two tiles along Mk: 1015-1257 us in order 5,
   // 772-862 us in order 3 (554 against 802, 561 against 769 us on two more); a seventh lost 9 %.
   if (opt.tiledOrder < 0 && neighbourRunsInMm) o.order = 3;
+  // ... and with every row on the 128-byte grid on both sides (no line is shared, the strips have nothing to keep
+  // together) such a plan walks the whole Mm axis at a stretch, order 1: 50 seeded plans of 0.3-0.8 GB per buffer in
+  // two sets (extents with and without powers of two, both widths, with and without Mbar ranks) ran +3.2 % in the
+  // mean against the strips, -1.8 % at worst; the tiles along Mk fastest +2 % (-6 ... +14 %), order 5 -0.5 %.
+  if (opt.superAuto && opt.tiledOrder < 0 && neighbourRunsInMm && beyondCache && rowBytesIn > 0 && rowBytesIn % 128 == 0 &&
+      rowBytesOut % 128 == 0)
+    o.order = 1;
   // One measured exception (forced-Tiled sweep over random shapes, all orders timed): with two
   // tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along Mk should run
   // fastest (order 2: 10-25 % faster), so that the thin tiles' few output rows are written as
