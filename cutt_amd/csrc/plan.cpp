@@ -776,7 +776,7 @@ int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK,
 
 int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
                     int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, bool mbarBetween,
-                    bool beyondCache, bool neighbourRunsInMm, TileOrdering& o, cuttHipTileDigits& dg) {
+                    bool beyondCache, bool neighbourRunsInMm, bool oneRankMk, TileOrdering& o, cuttHipTileDigits& dg) {
   std::memset(&dg, 0, sizeof(dg));
   if (!opt.tileDigits.empty()) {
     const int64_t logical = parseTileDigits(opt.tileDigits, tilesM, tilesK, volMbar, dg);
@@ -810,8 +810,9 @@ int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, i
   // together) such a plan walks the whole Mm axis at a stretch, order 1: 50 seeded plans of 0.3-0.8 GB per buffer in
   // two sets (extents with and without powers of two, both widths, with and without Mbar ranks) ran +3.2 % in the
   // mean against the strips, -1.8 % at worst; the tiles along Mk fastest +2 % (-6 ... +14 %), order 5 -0.5 %.
-  if (opt.superAuto && opt.tiledOrder < 0 && neighbourRunsInMm && beyondCache && rowBytesIn > 0 && rowBytesIn % 128 == 0 &&
-      rowBytesOut % 128 == 0)
+  // (All of those with a single rank along Mk; of two plans with a fused Mk axis one lost 10 %: left to the strips.)
+  if (opt.superAuto && opt.tiledOrder < 0 && neighbourRunsInMm && oneRankMk && beyondCache && rowBytesIn > 0 &&
+      rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0)
     o.order = 1;
   // One measured exception (forced-Tiled sweep over random shapes, all orders timed): with two
   // tiles along Mm of which the second is thin (a 65..88-wide rank), the tiles along Mk should run
@@ -1110,7 +1111,8 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     } else {
       plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
                                    sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache,
-                                   sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm, o, a.digits);
+                                   sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm, sp.numMk == 1, o,
+                                   a.digits);
     }
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     // How the kernels decode a free numbering.  Digit by digit costs a chain of up to 16 dependent scalar loads
@@ -1139,7 +1141,7 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     PlannerOptions copt = opt;
     copt.superAuto = false;  // (the measured exceptions are for the Tiled kernel only)
-    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, false, o, a.digits);
+    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, false, false, o, a.digits);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
