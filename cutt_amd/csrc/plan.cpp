@@ -774,9 +774,24 @@ int64_t parseTileDigits(const std::string& text, int64_t tilesM, int64_t tilesK,
   return logical;
 }
 
-int64_t tiledBlocks(const PlannerOptions& opt, int64_t tilesM, int64_t tilesK, int64_t volMbar,
-                    int64_t volMmLastTile, int64_t rowBytesIn, int64_t rowBytesOut, int elemSize, bool mbarBetween,
-                    bool beyondCache, bool neighbourRunsInMm, bool oneRankMk, TileOrdering& o, cuttHipTileDigits& dg) {
+// What the ordering rules of a tiled launch look at.
+struct TiledShape {
+  int64_t tilesM = 1, tilesK = 1, volMbar = 1;
+  int64_t volMmLastTile = kTile;            // elements along Mm in the last tile
+  int64_t rowBytesIn = 0, rowBytesOut = 0;  // bytes of one row of the Mm / Mk axis (0: not known, TiledCopy)
+  int elemSize = 4;
+  bool mbarBetween = false;        // an Mbar rank follows Mm in the input and Mk in the output
+  bool beyondCache = false;        // more than 0.75 memory-side cache sizes per buffer
+  bool neighbourRunsInMm = false;  // a fused Mm axis of which one rank follows Mk in the output
+  bool oneRankMk = false;          // a single rank along Mk
+};
+
+int64_t tiledBlocks(const PlannerOptions& opt, const TiledShape& shape, TileOrdering& o, cuttHipTileDigits& dg) {
+  const int64_t tilesM = shape.tilesM, tilesK = shape.tilesK, volMbar = shape.volMbar, volMmLastTile = shape.volMmLastTile;
+  const int64_t rowBytesIn = shape.rowBytesIn, rowBytesOut = shape.rowBytesOut;
+  const int elemSize = shape.elemSize;
+  const bool mbarBetween = shape.mbarBetween, beyondCache = shape.beyondCache, neighbourRunsInMm = shape.neighbourRunsInMm,
+             oneRankMk = shape.oneRankMk;
   std::memset(&dg, 0, sizeof(dg));
   if (!opt.tileDigits.empty()) {
     const int64_t logical = parseTileDigits(opt.tileDigits, tilesM, tilesK, volMbar, dg);
@@ -1109,10 +1124,19 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
         plan.numBlocks = (int64_t)o.xcdChunk * kNumXcd;
       }
     } else {
-      plan.numBlocks = tiledBlocks(opt, a.tilesM, a.tilesK, sp.volMbar, sp.volMm - (tilesM - 1) * kTile,
-                                   sp.volMm * pb.elemSize, sp.volMk * pb.elemSize, pb.elemSize, between, beyondCache,
-                                   sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm, sp.numMk == 1, o,
-                                   a.digits);
+      TiledShape shape;
+      shape.tilesM = a.tilesM;
+      shape.tilesK = a.tilesK;
+      shape.volMbar = sp.volMbar;
+      shape.volMmLastTile = sp.volMm - (tilesM - 1) * kTile;
+      shape.rowBytesIn = sp.volMm * pb.elemSize;
+      shape.rowBytesOut = sp.volMk * pb.elemSize;
+      shape.elemSize = pb.elemSize;
+      shape.mbarBetween = between;
+      shape.beyondCache = beyondCache;
+      shape.neighbourRunsInMm = sp.numMm > 1 && sp.numMk < pb.rank && pb.perm[sp.numMk] > 0 && pb.perm[sp.numMk] < sp.numMm;
+      shape.oneRankMk = sp.numMk == 1;
+      plan.numBlocks = tiledBlocks(opt, shape, o, a.digits);
     }
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     // How the kernels decode a free numbering.  Digit by digit costs a chain of up to 16 dependent scalar loads
@@ -1141,7 +1165,12 @@ bool setupTiled(Plan& plan, const cuttHipDeviceProps& props, const PlannerOption
     TileOrdering o;
     PlannerOptions copt = opt;
     copt.superAuto = false;  // (the measured exceptions are for the Tiled kernel only)
-    plan.numBlocks = tiledBlocks(copt, a.tilesM, a.tilesK, sp.volMbar, kTile, 0, 0, pb.elemSize, false, false, false, false, o, a.digits);
+    TiledShape shape;
+    shape.tilesM = a.tilesM;
+    shape.tilesK = a.tilesK;
+    shape.volMbar = sp.volMbar;
+    shape.elemSize = pb.elemSize;
+    plan.numBlocks = tiledBlocks(copt, shape, o, a.digits);
     a.order = o.order; a.xcdChunk = o.xcdChunk; a.superM = o.superM; a.superK = o.superK;
     a.cachePolicy = opt.cachePolicy;
     if (!fillMbar(pb, sp.inMmk, opt.mbarOrder, a.mbar)) return false;
