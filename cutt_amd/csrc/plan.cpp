@@ -849,10 +849,7 @@ int64_t tiledBlocks(const PlannerOptions& opt, const TiledShape& shape, TileOrde
   // a multiple of 16 KB: the 64 rows a tile reads then fall into few memory channels, and a band that spans the
   // whole of Mk has nothing else in flight (-8 ... -10 % at multiples of 32 and 64 KB); and not off the line
   // grid, where the tiles that share lines along Mm must run together (40 matrices: -6 % in the mean).
-  // Mbar ranks anywhere else than slowest: +4.2 % over 30 seeded plans (-10 ... +15 %); a rank between Mm and Mk
-  // (consecutive Mbar positions are neighbouring rows on both sides), against the patches and strips below: +1.9 %
-  // over 24 (-1.1 ... +9.5 %, both widths alike).
-  if (opt.superAuto && opt.tiledOrder < 0 && (o.order == 3 || o.order == 5) && !neighbourRunsInMm && beyondCache &&
+  if (opt.superAuto && opt.tiledOrder < 0 && (o.order == 3 || o.order == 5) && !mbarBetween && !neighbourRunsInMm && beyondCache &&
       rowBytesIn > 0 && rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0 && tilesM >= 16 && tilesK >= 17 && tilesK <= 700 &&
       rowBytesIn % 4096 != 0 && rowBytesIn % 16384 >= 1024 && rowBytesIn % 16384 <= 16384 - 1024)
     o.order = 2;

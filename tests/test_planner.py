@@ -230,8 +230,7 @@ def test_super_tile_shapes_of_the_tiled_plan(cutt):
     assert tiled((20480, 3392), (1, 0), 8)[0] == 3        # input rows a multiple of 4 KB apart
     assert tiled((8256, 16896), (1, 0), 4)[0] == 3        # ... and within 1 KB of a multiple of 16 KB
     assert tiled((4416, 25856), (1, 0), 4)[0] == 2
-    assert tiled((4416, 8, 12928), (2, 1, 0), 4)[0] == 2     # ... also with an Mbar rank between Mm and Mk
-    assert tiled((4608, 8, 12928), (2, 1, 0), 8) == (5, 2, 8)    # (input rows a multiple of 4 KB apart: patches)
+    assert tiled((4416, 8, 12928), (2, 1, 0), 4)[0] == 5     # an Mbar rank between Mm and Mk: not this rule
     assert tiled((2240, 2752), (1, 0), 8)[0] == 3         # inside the memory-side cache
 
 
