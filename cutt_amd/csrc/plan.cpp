@@ -849,6 +849,9 @@ int64_t tiledBlocks(const PlannerOptions& opt, const TiledShape& shape, TileOrde
   // a multiple of 16 KB: the 64 rows a tile reads then fall into few memory channels, and a band that spans the
   // whole of Mk has nothing else in flight (-8 ... -10 % at multiples of 32 and 64 KB); and not off the line
   // grid, where the tiles that share lines along Mm must run together (40 matrices: -6 % in the mean).
+  // Mbar ranks anywhere but between Mm and Mk: +4.2 % over 30 seeded plans of ranks 3-5 (-10 ... +15 %).  With a
+  // rank between, a band of 64 output rows is no contiguous piece; three seeded sets of such plans read +1.9 %,
+  // +5.5 % and -0.4 % (-15 % at worst) against the patches and strips below, which they keep.
   if (opt.superAuto && opt.tiledOrder < 0 && (o.order == 3 || o.order == 5) && !mbarBetween && !neighbourRunsInMm && beyondCache &&
       rowBytesIn > 0 && rowBytesIn % 128 == 0 && rowBytesOut % 128 == 0 && tilesM >= 16 && tilesK >= 17 && tilesK <= 700 &&
       rowBytesIn % 4096 != 0 && rowBytesIn % 16384 >= 1024 && rowBytesIn % 16384 <= 16384 - 1024)
