@@ -50,9 +50,11 @@ def test_sweep_both_planners_every_tensor():
     assert worst_measured["measure"]["pct"] >= 70.0, worst_measured
     assert worst_heuristic["plan"]["pct"] >= 70.0, worst_heuristic
     # the measuring planner must not end up behind the heuristic one by more than timing noise (the two plans are
-    # timed in turn, the best of four runs each)
+    # timed in turn, the best of four runs each; the planner's own last comparison of the two is the best of two)
     for r in results:
-        assert r["measure"]["ms"] <= 1.05 * r["plan"]["ms"], r
+        assert r["measure"]["ms"] <= 1.08 * r["plan"]["ms"], r
+    behind = [r["measure"]["ms"] / r["plan"]["ms"] for r in results]
+    assert float(np.mean(behind)) <= 1.0, behind
 
 
 @pytest.mark.parametrize("index", [0, 9, 18, 27, 36, 45])
