@@ -63,6 +63,8 @@ def timed_pair(cfg, env_off, reps=4, launches=3):
     return gb / best["on"], gb / best["off"], infos["on"], infos["off"]
 
 
+# The floors of these checks leave room for the timing noise of a fresh machine: a single plan's ratio moves by
+# 2-3 % from run to run (the lowest of eight by up to 5 %), a mean over eight by about 1 %.
 def run_rule(name, cases, env_off, applies, mean_floor, min_floor, need):
     import torch
     assert torch.cuda.is_available(), "this test needs the MI355X"
@@ -102,7 +104,7 @@ def test_workgroups_numbered_by_address_bits():
     # batched transposes on power-of-two addresses (other extents than the tensors the rule was derived on: last
     # rank 5 and 6, both widths); found: +8 % in the mean over 35 + 36 such tensors
     run_rule("address bits (Tiled)", pow2_batched(2027, 10), {"CUTT_ADDRESS_BITS": "0"},
-             lambda on, off: on.method_name == "Tiled" and on.tiledOrder == 7, 1.02, 0.95, 6)
+             lambda on, off: on.method_name == "Tiled" and on.tiledOrder == 7, 1.02, 0.90, 6)
 
 
 def test_packed_items_with_address_bit_11_moving():
@@ -132,7 +134,7 @@ def test_packed_items_with_address_bit_11_moving():
                 cases.append(dict(dim=dim, perm=perm, es=es))
     assert len(cases) == 12, tries
     run_rule("address bit 11 (packed)", cases, {"CUTT_ADDRESS_BITS": "0"},
-             lambda on, off: bool(on.tileDigits) and on.method_name == off.method_name, 0.97, 0.82, 8)
+             lambda on, off: bool(on.tileDigits) and on.method_name == off.method_name, 0.96, 0.78, 8)
 
 
 def test_run_length_term_of_the_model_for_runs_on_the_line_grid(monkeypatch):
@@ -170,7 +172,7 @@ def test_run_length_term_of_the_model_for_runs_on_the_line_grid(monkeypatch):
             cases.append(dict(dim=dim, perm=perm, es=es))
     assert len(cases) == 14, tries
     run_rule("run lengths on the line grid (model)", cases, {"CUTT_MODEL_RUN_LENGTH": "0"},
-             lambda on, off: True, 1.0, 0.82, 10)
+             lambda on, off: True, 0.99, 0.82, 10)
 
 
 def test_tiles_over_fused_rank_sets():
@@ -187,7 +189,7 @@ def test_tiles_over_fused_rank_sets():
             continue
         cases.append(dict(dim=tuple(dim), perm=tuple(perm), es=8 if len(cases) % 2 == 0 else 4))
     run_rule("tiles over fused rank sets", cases, {"CUTT_TILED_FUSE": "0"},
-             lambda on, off: on.method_name == "Tiled" and (on.numMm > 1 or on.numMk > 1), 1.02, 0.93, 3)
+             lambda on, off: on.method_name == "Tiled" and (on.numMm > 1 or on.numMk > 1), 1.02, 0.90, 3)
 
 
 def test_strips_sixteen_wide_for_rows_32_kb_apart():
@@ -199,7 +201,7 @@ def test_strips_sixteen_wide_for_rows_32_kb_apart():
         rows = int(rng.integers(6500, 12000))
         cases.append(dict(dim=(8192 * n, rows // n), perm=(1, 0), es=4))
     run_rule("16-wide strips", cases, {"CUTT_SUPER_M": "8"},
-             lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.superM == 16, 1.03, 0.98, 4)
+             lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.superM == 16, 1.03, 0.95, 4)
 
 
 def test_rows_in_groups_for_unaligned_four_byte_rows():
@@ -214,7 +216,7 @@ def test_rows_in_groups_for_unaligned_four_byte_rows():
         cases.append(dict(dim=(a, b, c), perm=(2, 1, 0), es=4))
     run_rule("rows in groups", cases, {"CUTT_TILED_GROUPED": "0"},
              lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.tiledGrouped == 1 and off.tiledGrouped == 0,
-             1.0, 0.95, 4)
+             1.0, 0.93, 4)
 
 
 def test_patches_for_eight_byte_rows_on_the_line_grid():
@@ -258,7 +260,7 @@ def test_one_strip_for_a_rank_of_nine_to_fourteen_tiles():
     # (46 such plans: +2 % in the mean, single ones -7 ... +16 %)
     run_rule("one strip", cases, {"CUTT_SUPER_M": "8"},
              lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.superM > 8 and on.numMm == 1,
-             0.995, 0.91, 8)
+             0.995, 0.88, 8)
 
 
 def test_thin_second_tile_lets_the_tiles_along_mk_run_fastest():
@@ -328,7 +330,7 @@ def test_whole_mm_axis_at_a_stretch_for_fused_mm_sets_on_the_line_grid():
         cases.append(dict(dim=dim, perm=perm, es=es))
     run_rule("whole Mm axis at a stretch", cases, {"CUTT_TILED_ORDER": "3"},
              lambda on, off: on.method_name == "Tiled" and off.method_name == "Tiled" and on.numMm > 1 and on.tiledOrder == 1,
-             1.0, 0.95, 5)
+             0.99, 0.95, 5)
 
 
 def test_work_items_per_workgroup_and_their_order():
@@ -405,7 +407,7 @@ def test_order_of_the_mbar_ranks():
         cases.append(dict(dim=tuple(dim), perm=tuple(perm), es=8 if len(cases) % 2 == 0 else 4))
     run_rule("Mbar order", cases, {"CUTT_MBAR_ORDER": "2"},
              lambda on, off: abs(on.usPredicted - off.usPredicted) > 1e-6 * off.usPredicted or on.method_name != off.method_name,
-             0.98, 0.90, 3)   # (13 changed plans of 150 random tensors: +1.9 % in the mean, -1 ... +9 %)
+             0.97, 0.90, 3)   # (13 changed plans of 150 random tensors: +1.9 % in the mean, -1 ... +9 %)
 
 
 def test_strips_per_mbar_position_for_fused_mm_sets():
